@@ -1,0 +1,267 @@
+// Token dispatch and combine for gfx950.
+//
+// Replaces moe_expert_count, which the reference runs on the CPU between two blocking copies
+// (plugin/cuda/moe.cu:161-212), by three small device kernels with no host round trip:
+//   1. per-block histogram of the expert assignment,
+//   2. one-workgroup exclusive scan over (block, expert) and over experts, which also emits the
+//      row tiles of the grouped expert launch,
+//   3. stable ranking: token t goes to row offset[e] + (tokens of e in earlier blocks) +
+//      (tokens of e earlier in this block).  The rank inside a block is built from wave ballots
+//      in token order, so the permutation does not depend on the order atomics retire in and is
+//      bit-identical to the reference's sequential counting sort.
+// and the row-copy kernels batch_scatter_feature_and_weight_kernel / batch_gather_kernel /
+// fused_batch_mix_and_gather_kernel (plugin/cuda/moe.cu:89-127) by wave-per-row copies with
+// 16-byte accesses.
+#include <hip/hip_runtime.h>
+
+#include <initializer_list>
+
+#include "kernels.h"
+
+namespace infmoe {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+constexpr int kThreads = 256;
+constexpr int kPerThread = kCountBlockTokens / kThreads;
+
+__global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int* __restrict__ sel,
+                                                        int* __restrict__ blockhist) {
+    extern __shared__ int s_hist[];
+    for (int e = threadIdx.x; e < E; e += kThreads) s_hist[e] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * kCountBlockTokens;
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+        const int t = base + j * kThreads + threadIdx.x;
+        if (t < T) atomicAdd(&s_hist[min(max(sel[t], 0), E - 1)], 1);  // integer sums: order-free
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += kThreads) blockhist[(size_t)blockIdx.x * E + e] = s_hist[e];
+}
+
+__global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, int* __restrict__ blockhist,
+                                                        int* __restrict__ count, int* __restrict__ offset,
+                                                        RowTile* __restrict__ tiles, int* __restrict__ n_tiles,
+                                                        int tile_rows, int skinny_max) {
+    for (int e = threadIdx.x; e < E; e += kThreads) {
+        int run = 0;
+        for (int b = 0; b < nblk; ++b) {
+            const int c = blockhist[(size_t)b * E + e];
+            blockhist[(size_t)b * E + e] = run;  // tokens of e in earlier blocks
+            run += c;
+        }
+        count[e] = run;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int off = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            const int c = count[e];
+            offset[e] = off;
+            if (tiles != nullptr && c > skinny_max) {
+                for (int m0 = 0; m0 < c; m0 += tile_rows) {
+                    RowTile rt;
+                    rt.expert = e;
+                    rt.row0 = off + m0;
+                    rt.rows = min(tile_rows, c - m0);
+                    rt.pad = 0;
+                    tiles[nt++] = rt;
+                }
+            }
+            off += c;
+        }
+        offset[E] = off;  // == T (plugin/MoELayerPlugin.cc:351)
+        if (n_tiles != nullptr) *n_tiles = nt;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void rank_kernel(int T, int E, const int* __restrict__ sel,
+                                                        const int* __restrict__ blockbase,
+                                                        const int* __restrict__ offset, int* __restrict__ pos,
+                                                        int* __restrict__ row_expert) {
+    extern __shared__ int s_run[];  // tokens of each expert already ranked in this block
+    for (int e = threadIdx.x; e < E; e += kThreads) s_run[e] = offset[e] + blockbase[(size_t)blockIdx.x * E + e];
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int base = blockIdx.x * kCountBlockTokens;
+    for (int j = 0; j < kPerThread; ++j) {
+        const int t = base + j * kThreads + threadIdx.x;  // token order == (j, wave, lane) order
+        const bool valid = t < T;
+        const int e = valid ? min(max(sel[t], 0), E - 1) : -1;
+        // rank among the lanes of this wave that chose the same expert
+        int rank = 0, cnt = 0;
+        bool leader = false;
+        unsigned long long todo = __ballot(valid);
+        while (todo) {
+            const int first = __ffsll((long long)todo) - 1;
+            const int ef = __shfl(e, first);
+            const unsigned long long same = __ballot(valid && e == ef);
+            if (e == ef) {
+                rank = __popcll(same & below);
+                cnt = __popcll(same);
+                leader = (lane == first);
+            }
+            todo &= ~same;
+        }
+        // waves take turns so that earlier tokens get lower rows
+        for (int w = 0; w < kThreads / 64; ++w) {
+            if (wave == w && valid) {
+                const int r = s_run[e] + rank;
+                pos[r] = t;
+                if (row_expert != nullptr) row_expert[r] = e;
+            }
+            __syncthreads();
+            if (wave == w && leader) s_run[e] += cnt;
+            __syncthreads();
+        }
+    }
+}
+
+// ---- row copies: one wave per row, 16-byte accesses when the row length allows
+template <bool VEC>
+__device__ __forceinline__ void copy_row(float* __restrict__ dst, const float* __restrict__ src, int d, int lane) {
+    if (VEC) {
+        const int n4 = d >> 2;
+        const v4f* s = reinterpret_cast<const v4f*>(src);
+        v4f* o = reinterpret_cast<v4f*>(dst);
+        int k = lane;
+        for (; k + 192 < n4; k += 256) {  // four independent loads in flight
+            const v4f a = s[k], b = s[k + 64], c = s[k + 128], e = s[k + 192];
+            o[k] = a;
+            o[k + 64] = b;
+            o[k + 128] = c;
+            o[k + 192] = e;
+        }
+        for (; k < n4; k += 64) o[k] = s[k];
+    } else {
+        for (int k = lane; k < d; k += 64) dst[k] = src[k];
+    }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void scatter_kernel(int T, int d, const float* __restrict__ x,
+                                                           const float* __restrict__ coeff,
+                                                           const int* __restrict__ pos, float* __restrict__ routed,
+                                                           float* __restrict__ routed_coeff) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (r >= T) return;
+    const int t = pos[r];
+    copy_row<VEC>(routed + (size_t)r * d, x + (size_t)t * d, d, lane);
+    if (lane == 0 && coeff != nullptr && routed_coeff != nullptr) routed_coeff[r] = coeff[t];
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void gather_kernel(int T, int d, const float* __restrict__ buf,
+                                                          const int* __restrict__ pos, float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (r >= T) return;
+    copy_row<VEC>(out + (size_t)pos[r] * d, buf + (size_t)r * d, d, lane);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void mix_gather_kernel(int T, int d, const int* __restrict__ pos,
+                                                              const float* __restrict__ routed,
+                                                              const float* __restrict__ post,
+                                                              const float* __restrict__ routed_coeff,
+                                                              float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (r >= T) return;
+    // plugin/cuda/common.cuh:24-27 and plugin/cuda/moe.cu:120-126
+    const float a = 1.0f / (1.0f + expf(-routed_coeff[r]));
+    const float b = 1.0f - a;
+    const float* p = post + (size_t)r * d;
+    const float* q = routed + (size_t)r * d;
+    float* o = out + (size_t)pos[r] * d;
+    if (VEC) {
+        const int n4 = d >> 2;
+        const v4f* p4 = reinterpret_cast<const v4f*>(p);
+        const v4f* q4 = reinterpret_cast<const v4f*>(q);
+        v4f* o4 = reinterpret_cast<v4f*>(o);
+        int k = lane;
+        for (; k + 64 < n4; k += 128) {
+            const v4f p0 = p4[k], p1 = p4[k + 64], q0 = q4[k], q1 = q4[k + 64];
+            o4[k] = a * p0 + b * q0;
+            o4[k + 64] = a * p1 + b * q1;
+        }
+        for (; k < n4; k += 64) o4[k] = a * p4[k] + b * q4[k];
+    } else {
+        for (int k = lane; k < d; k += 64) o[k] = a * p[k] + b * q[k];
+    }
+}
+
+__global__ void fill_i32_kernel(int* __restrict__ dst, int n, int value) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = value;
+}
+
+inline dim3 row_grid(int T) { return dim3((T + kThreads / 64 - 1) / (kThreads / 64)); }
+
+// 16-byte accesses need rows that start on 16-byte boundaries
+inline bool vec_ok(int d, std::initializer_list<const void*> ptrs) {
+    if (d % 4 != 0) return false;
+    for (const void* p : ptrs)
+        if (reinterpret_cast<uintptr_t>(p) & 15) return false;
+    return true;
+}
+
+}  // namespace
+
+size_t expert_count_scratch_bytes(int T, int E) {
+    const size_t nblk = (size_t)(T + kCountBlockTokens - 1) / kCountBlockTokens;
+    return ((nblk * (size_t)E * sizeof(int)) + 255) & ~(size_t)255;
+}
+
+hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
+                               RowTile* tiles, int* n_tiles, int tile_rows, int skinny_max, int* row_expert,
+                               hipStream_t stream) {
+    const int nblk = (T + kCountBlockTokens - 1) / kCountBlockTokens;
+    int* blockhist = static_cast<int*>(scratch);
+    const size_t lds = (size_t)E * sizeof(int);
+    if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
+    scan_kernel<<<1, kThreads, 0, stream>>>(T, E, nblk, blockhist, count, offset, tiles, n_tiles, tile_rows,
+                                            skinny_max);
+    if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream) {
+    if (n <= 0) return hipSuccess;
+    fill_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, n, value);
+    return hipGetLastError();
+}
+
+hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, const int* pos, float* routed,
+                          float* routed_coeff, hipStream_t stream) {
+    if (T <= 0) return hipSuccess;
+    if (vec_ok(d, {x, routed}))
+        scatter_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, x, coeff, pos, routed, routed_coeff);
+    else
+        scatter_kernel<false><<<row_grid(T), kThreads, 0, stream>>>(T, d, x, coeff, pos, routed, routed_coeff);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream) {
+    if (T <= 0) return hipSuccess;
+    if (vec_ok(d, {buf, out}))
+        gather_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out);
+    else
+        gather_kernel<false><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_mix_gather(int T, int d, const int* pos, const float* routed, const float* post,
+                             const float* routed_coeff, float* out, hipStream_t stream) {
+    if (T <= 0) return hipSuccess;
+    if (vec_ok(d, {routed, post, out}))
+        mix_gather_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, pos, routed, post, routed_coeff, out);
+    else
+        mix_gather_kernel<false><<<row_grid(T), kThreads, 0, stream>>>(T, d, pos, routed, post, routed_coeff, out);
+    return hipGetLastError();
+}
+
+}  // namespace infmoe

@@ -1,0 +1,88 @@
+// Host-side launchers of the gfx950 kernels.  Plain C++ signatures (no HIP kernel syntax) so
+// the host code of the layer and of the sub-layers can be read without the device code.
+// Every launcher is asynchronous on `stream` and returns the hipError_t of the launch.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace infmoe {
+
+enum NormKind : int32_t { NORM_NONE = 0, NORM_RMS = 1, NORM_CENTERED = 2 };
+enum FfnKind : int32_t { FFN_RELU = 0, FFN_GATED_GELU = 1 };
+
+constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/sublayers/T5FFLayer.cc:102
+
+// ---- gating (replaces layernorm_gpu + cublasSgemm + expert_select_top1_kernel,
+//      plugin/MoELayerPlugin.cc:315-345)
+hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
+                            int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
+                            hipStream_t stream);
+
+// ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)
+// Row tile of the grouped expert GEMM: `rows` consecutive routed rows of one expert.
+struct RowTile {
+    int32_t expert;
+    int32_t row0;  // first routed row
+    int32_t rows;  // 1..tile height
+    int32_t pad;
+};
+constexpr int kCountBlockTokens = 1024;  // tokens ranked by one workgroup
+size_t expert_count_scratch_bytes(int T, int E);
+// Optional outputs for the grouped expert launch (all may be null):
+//   tiles/n_tiles: row tiles of height <= tile_rows over experts with more than `skinny_max` rows
+//   row_expert[T]: expert of every routed row
+hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
+                               RowTile* tiles, int* n_tiles, int tile_rows, int skinny_max, int* row_expert,
+                               hipStream_t stream);
+inline int max_row_tiles(int T, int E, int tile_rows) { return (T + tile_rows - 1) / tile_rows + E; }
+
+// Small fill kernel (used instead of hipMemsetAsync so that callers may capture the layer in a graph).
+hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream);
+
+// ---- scatter / gather / mix (replaces plugin/cuda/moe.cu:214-258)
+hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, const int* pos, float* routed,
+                          float* routed_coeff, hipStream_t stream);
+hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream);
+hipError_t launch_mix_gather(int T, int d, const int* pos, const float* routed, const float* post,
+                             const float* routed_coeff, float* out, hipStream_t stream);
+
+// ---- row norm (replaces layernorm_gpu, plugin/cuda/ops/layernorm.cu:176-188)
+// gamma of row r is gamma_base + row_expert[r] * gamma_stride (row_expert null -> gamma_base).
+hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const float* gamma_base,
+                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream);
+
+// ---- expert GEMMs (replace the three cublasSgemm_v2 calls, fused_gelu_dot_gpu and the D2D
+//      residual copy of plugin/sublayers/T5FFLayer.cc:112-138)
+enum Epilogue : int32_t {
+    EPI_RELU = 0,        // C = max(A*B^T, 0)
+    EPI_GATED_GELU = 1,  // C = gelu_tanh(A*B0^T) * (A*B1^T)
+    EPI_RESIDUAL = 2     // C = R + A*B^T
+};
+struct GemmProblem {
+    const float* A;    // [rows][K] activations (row stride K)
+    const float* B;    // [N][K] weights, K contiguous (torch Linear layout)
+    const float* B1;   // second weight matrix for EPI_GATED_GELU, else null
+    const float* R;    // [rows][N] residual for EPI_RESIDUAL, else null
+    float* C;          // [rows][N]
+    int N, K;
+    int epilogue;
+};
+// One expert, `rows` known on the host.
+hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream);
+// All experts in one launch: A, R, C address routed rows globally; expert e's weights are at
+// B + e*weight_stride (floats).  Row tiles and their number come from launch_expert_count.
+hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
+                                      const int* n_tiles, int max_tiles, hipStream_t stream);
+constexpr int kGemmTileRows = 256;  // tallest row tile of the GEMM kernel
+
+// Few-row experts (decode): every weight row is streamed once and dotted with up to
+// kSkinnyMaxRows activation rows held in LDS.
+constexpr int kSkinnyMaxRows = 8;
+hipError_t launch_expert_skinny(const GemmProblem& p, int rows, hipStream_t stream);
+hipError_t launch_expert_skinny_grouped(const GemmProblem& p, size_t weight_stride, const int* count,
+                                        const int* offset, int E, hipStream_t stream);
+
+}  // namespace infmoe

@@ -1,0 +1,104 @@
+// Row norm with gamma only (the reference calls layernorm_gpu with beta == nullptr at both sites,
+// plugin/MoELayerPlugin.cc:324-325 and plugin/sublayers/T5FFLayer.cc:102-103).
+//   centered: gamma * (x - mu) * rsqrt(var + eps), biased variance  (plugin/cuda/ops/layernorm.cu:149-161)
+//   rms:      gamma * x * rsqrt(mean(x^2) + eps)                    (README.md:115)
+// One wave per row.  The row is read once into registers when it is at most 8192 floats (two
+// exact passes for the centered form: mean, then variance about the mean, instead of the
+// reference's Welford merge) and re-read from cache otherwise.  For the grouped expert launch
+// every routed row picks the gamma of its own expert.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace infmoe {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+constexpr int kThreads = 256;
+constexpr int kRegVec = 32;  // float4 per lane held in registers -> rows up to 64*32*4 = 8192 floats
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                            int rows, int d, const float* __restrict__ gamma_base,
+                                                            size_t gamma_stride, const int* __restrict__ row_expert,
+                                                            int norm_kind) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const float* x = in + (size_t)r * d;
+    float* y = out + (size_t)r * d;
+    const float* g = gamma_base + (row_expert ? (size_t)row_expert[r] * gamma_stride : 0);
+    const float inv_d = 1.0f / (float)d;
+
+    if (VEC && d <= 64 * 4 * kRegVec) {
+        const int n4 = d >> 2;
+        v4f v[kRegVec];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < kRegVec; ++j) {
+            const int k = lane + 64 * j;
+            v[j] = (k < n4) ? reinterpret_cast<const v4f*>(x)[k] : v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        float mu = 0.f;
+        if (norm_kind == NORM_CENTERED) {
+#pragma unroll
+            for (int j = 0; j < kRegVec; ++j) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+            mu = wave_sum(s) * inv_d;
+        }
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < kRegVec; ++j) {
+            const int k = lane + 64 * j;
+            if (k < n4) {
+                const v4f c = v[j] - mu;
+                q += (c.x * c.x + c.y * c.y) + (c.z * c.z + c.w * c.w);
+            }
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_d + kNormEps);
+#pragma unroll
+        for (int j = 0; j < kRegVec; ++j) {
+            const int k = lane + 64 * j;
+            if (k < n4) reinterpret_cast<v4f*>(y)[k] = reinterpret_cast<const v4f*>(g)[k] * ((v[j] - mu) * rstd);
+        }
+    } else {
+        float mu = 0.f;
+        if (norm_kind == NORM_CENTERED) {
+            float s = 0.f;
+            for (int k = lane; k < d; k += 64) s += x[k];
+            mu = wave_sum(s) * inv_d;
+        }
+        float q = 0.f;
+        for (int k = lane; k < d; k += 64) {
+            const float c = x[k] - mu;
+            q += c * c;
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_d + kNormEps);
+        for (int k = lane; k < d; k += 64) y[k] = g[k] * ((x[k] - mu) * rstd);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const float* gamma_base,
+                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream) {
+    if (rows <= 0) return hipSuccess;
+    const dim3 grid((rows + kThreads / 64 - 1) / (kThreads / 64));
+    const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in) |
+                           reinterpret_cast<uintptr_t>(gamma_base)) & 15) == 0 &&
+                         (gamma_stride % 4 == 0);
+    if (d % 4 == 0 && aligned)
+        row_norm_kernel<true><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert,
+                                                             norm_kind);
+    else
+        row_norm_kernel<false><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert,
+                                                              norm_kind);
+    return hipGetLastError();
+}
+
+}  // namespace infmoe

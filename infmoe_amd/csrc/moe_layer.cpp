@@ -1,0 +1,418 @@
+#include "moe_layer.h"
+
+#include <sys/stat.h>
+
+#include <algorithm>
+#include <cstring>
+
+namespace infmoe {
+
+std::string& last_error_slot() {
+    static thread_local std::string slot;
+    return slot;
+}
+
+// ---------------------------------------------------------------- construction
+
+Status MoELayer::parseFlags(const char* variant, MoEFlags* out) {
+    // plugin/MoELayerPlugin.cc:44-58, names from plugin/MoELayerPlugin.h:28-32
+    MoEFlags f;
+    if (variant == nullptr) return fail(INFMOE_ERR_MISSING_FIELD, "moe_variant is required");
+    if (strcmp(variant, "base_layer") == 0) {
+        f.baseLayerOutputMix = true;
+    } else if (strcmp(variant, "cpm_2") == 0) {
+        f.layernormOnInputBeforeScore = true;
+    } else if (strcmp(variant, "default") == 0) {
+    } else {
+        return fail(INFMOE_ERR_UNSUPPORTED, "unsupported moe variant: %s", variant);
+    }
+    *out = f;
+    return INFMOE_OK;
+}
+
+Status MoELayer::create(MoEParams&& p, std::unique_ptr<MoELayer>* out) {
+    // plugin/MoELayerPluginCreator.cc:117-140 and plugin/MoELayerPlugin.cc:74-80
+    if (p.embeddingSize <= 0) return fail(INFMOE_ERR_MISSING_FIELD, "embedding_size must be given and positive");
+    if (p.expertCount <= 0) return fail(INFMOE_ERR_MISSING_FIELD, "expert_count must be given and positive");
+    if (p.hiddenSize <= 0) return fail(INFMOE_ERR_MISSING_FIELD, "hidden_size must be given and positive");
+    if (p.maxConcurrency <= 0) return fail(INFMOE_ERR_INVALID_ARGUMENT, "max_concurrency must be positive");
+    if (p.centroids.empty()) return fail(INFMOE_ERR_MISSING_FIELD, "expert_centroids is required");
+    if (p.centroids.size() != (size_t)p.embeddingSize * p.expertCount)
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "expert_centroids has %zu floats, expected expert_count*embedding_size = %zu",
+                    p.centroids.size(), (size_t)p.embeddingSize * p.expertCount);
+    if (p.sublayerType.empty()) return fail(INFMOE_ERR_MISSING_FIELD, "expert_sublayer_type is required");
+    if (p.variant.empty()) return fail(INFMOE_ERR_MISSING_FIELD, "moe_variant is required");
+    if (!p.layernormWeight.empty() && p.layernormWeight.size() != (size_t)p.embeddingSize)
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "layernorm_weight has %zu floats, expected embedding_size = %d",
+                    p.layernormWeight.size(), p.embeddingSize);
+    INFMOE_TRY(parseFlags(p.variant.c_str(), &p.flags));
+    if (p.flags.layernormOnInputBeforeScore && p.layernormWeight.empty())
+        return fail(INFMOE_ERR_MISSING_FIELD, "layernorm_weight is required for moe_variant cpm_2");
+    if (!p.weightFile.empty()) {
+        struct stat st {};
+        if (stat(p.weightFile.c_str(), &st) != 0) return fail(INFMOE_ERR_IO, "cannot stat weight file: %s", p.weightFile.c_str());
+        if (!S_ISREG(st.st_mode)) return fail(INFMOE_ERR_IO, "weight file must be a regular file: %s", p.weightFile.c_str());
+    }
+    std::unique_ptr<MoELayer> layer(new MoELayer());
+    INFMOE_TRY(make_sublayer(p.sublayerType.c_str(), p.expertCount, p.embeddingSize, p.hiddenSize,
+                             p.weightFile.empty() ? nullptr : p.weightFile.c_str(), p.maxConcurrency, p.normKind,
+                             p.ffnKind, &layer->mSublayer));
+    layer->mParams = std::move(p);
+    *out = std::move(layer);
+    return INFMOE_OK;
+}
+
+Status MoELayer::clone(std::unique_ptr<MoELayer>* out) const {
+    std::unique_ptr<MoELayer> layer(new MoELayer());
+    layer->mParams = mParams;       // deep copy of centroids / gamma
+    layer->mSublayer = mSublayer;   // shared, so stacked layers hold the expert weights once
+    layer->mScoreBias = mScoreBias;
+    layer->mSequenceLength = mSequenceLength;
+    *out = std::move(layer);
+    return INFMOE_OK;
+}
+
+MoELayer::~MoELayer() { (void)terminate(); }
+
+Status MoELayer::setScoreBias(const float* host) {
+    if (host == nullptr) {
+        mScoreBias.clear();
+    } else {
+        mScoreBias.assign(host, host + mParams.expertCount);
+    }
+    if (mInitialized) {
+        if (mScoreBias.empty()) return INFMOE_OK;
+        if (mScoreBiasGpu == nullptr) INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mScoreBiasGpu), sizeof(float) * mParams.expertCount));
+        INFMOE_HIP(hipMemcpy(mScoreBiasGpu, mScoreBias.data(), sizeof(float) * mParams.expertCount, hipMemcpyHostToDevice));
+    }
+    return INFMOE_OK;
+}
+
+// ---------------------------------------------------------------- shapes and workspace
+
+Status MoELayer::checkDims(const int32_t* dims, int32_t nbDims, int* tokens) const {
+    // plugin/MoELayerPlugin.cc:172-177
+    if (dims == nullptr || nbDims != 3) return fail(INFMOE_ERR_INVALID_ARGUMENT, "input must be 3-D [batch, seq, embedding_size]");
+    if (dims[2] != mParams.embeddingSize)
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "last input dimension is %d, expected embedding_size = %d", dims[2], mParams.embeddingSize);
+    if (dims[0] < 0 || dims[1] < 0) return fail(INFMOE_ERR_INVALID_ARGUMENT, "negative input dimension");
+    const int64_t t = (int64_t)dims[0] * dims[1];
+    if (t > 0x3fffffff) return fail(INFMOE_ERR_INVALID_ARGUMENT, "too many tokens");
+    *tokens = (int)t;
+    return INFMOE_OK;
+}
+
+Status MoELayer::configure(const int32_t* dims, int32_t nbDims) {
+    int t = 0;
+    INFMOE_TRY(checkDims(dims, nbDims, &t));
+    Dims in;
+    in.nbDims = 3;
+    for (int i = 0; i < 3; ++i) in.d[i] = dims[i];
+    if (!mSublayer->configureWithFormat(&in, 1, &in, 1)) return fail(INFMOE_ERR_INVALID_ARGUMENT, "sub-layer rejected the input format");
+    mSequenceLength = dims[1];
+    return INFMOE_OK;
+}
+
+bool MoELayer::resident() const {
+    return mSublayer->weightSize() == 0 || mParams.maxConcurrency >= mParams.expertCount;
+}
+
+struct MoELayer::Carve {
+    char* slots = nullptr;
+    size_t slotStride = 0;
+    char* subWs = nullptr;
+    int32_t *sel = nullptr, *pos = nullptr, *rowExpert = nullptr, *nTiles = nullptr;
+    RowTile* tiles = nullptr;
+    int maxTiles = 0;
+    void* countScratch = nullptr;
+    float *coeff = nullptr, *routedCoeff = nullptr, *routed = nullptr, *post = nullptr;
+    size_t total = 0;
+};
+
+// Workspace layout (every block 256-byte aligned):
+//   streamed experts only: max_concurrency weight slots           (plugin/MoELayerPlugin.cc:243-245)
+//   sub-layer scratch for T rows, shared by all experts because their rows are disjoint
+//     (the reference sizes one full-T scratch per slot, :256-263)
+//   sel[T] pos[T] rowExpert[T] | row tiles | scan scratch | coeff[T] routedCoeff[T] | routed[T][d] | post[T][d]
+//   (the reference also keeps the T x E score matrix, :246; the fused gating never stores it)
+Status MoELayer::carve(int T, void* workspace, Carve* c) const {
+    char* base = static_cast<char*>(workspace);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* p = base ? base + off : nullptr;
+        off += align_up(bytes);
+        return p;
+    };
+    const int E = mParams.expertCount, d = mParams.embeddingSize;
+    c->slotStride = align_up(mSublayer->weightSize());
+    c->slots = resident() ? nullptr : take(c->slotStride * (size_t)mParams.maxConcurrency);
+    c->subWs = take(mSublayer->workspaceSize(T));
+    c->sel = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
+    c->pos = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
+    c->rowExpert = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
+    c->maxTiles = max_row_tiles(T, E, kGemmTileRows);
+    c->tiles = reinterpret_cast<RowTile*>(take(sizeof(RowTile) * (size_t)c->maxTiles));
+    c->nTiles = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
+    c->countScratch = take(expert_count_scratch_bytes(T, E));
+    c->coeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
+    c->routedCoeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
+    c->routed = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T * d));
+    c->post = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T * d));
+    c->total = off;
+    return INFMOE_OK;
+}
+
+Status MoELayer::workspaceSize(const int32_t* dims, int32_t nbDims, size_t* bytes) const {
+    int T = 0;
+    INFMOE_TRY(checkDims(dims, nbDims, &T));
+    if (bytes == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null output pointer");
+    Carve c;
+    INFMOE_TRY(carve(T, nullptr, &c));
+    *bytes = c.total;
+    return INFMOE_OK;
+}
+
+// ---------------------------------------------------------------- initialize / terminate
+
+Status MoELayer::initialize() {
+    if (mInitialized) return INFMOE_OK;
+    const int E = mParams.expertCount, d = mParams.embeddingSize;
+    INFMOE_TRY(mSublayer->initialize());
+    // plugin/MoELayerPlugin.cc:14-26 (done on the first enqueue there)
+    INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mCentroidsGpu), sizeof(float) * (size_t)E * d));
+    INFMOE_HIP(hipMemcpy(mCentroidsGpu, mParams.centroids.data(), sizeof(float) * (size_t)E * d, hipMemcpyHostToDevice));
+    if (!mParams.layernormWeight.empty()) {
+        INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mLayernormGpu), sizeof(float) * d));
+        INFMOE_HIP(hipMemcpy(mLayernormGpu, mParams.layernormWeight.data(), sizeof(float) * d, hipMemcpyHostToDevice));
+    }
+    const size_t routingInts = (size_t)2 * E + 1 + 4;
+    INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mRoutingGpu), sizeof(int32_t) * routingInts));
+    INFMOE_HIP(hipMemset(mRoutingGpu, 0, sizeof(int32_t) * routingInts));
+    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mRoutingHost), sizeof(int32_t) * routingInts, hipHostMallocDefault));
+    INFMOE_HIP(hipEventCreateWithFlags(&mRoutingDone, hipEventDisableTiming));
+    if (resident()) {
+        INFMOE_TRY(mSublayer->makeResident());
+    } else {
+        // plugin/MoELayerPlugin.cc:182-195 creates max_concurrency streams; here one copy stream
+        // feeds the slots and a few compute streams let consecutive experts overlap
+        INFMOE_HIP(hipStreamCreateWithFlags(&mCopyStream, hipStreamNonBlocking));
+        mComputeStreams.resize(std::min(mParams.maxConcurrency, 4));
+        for (auto& s : mComputeStreams) INFMOE_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+        mJoin.resize(mComputeStreams.size());
+        for (auto& e : mJoin) INFMOE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        mCopyDone.resize(E);
+        mComputeDone.resize(E);
+        for (auto& e : mCopyDone) INFMOE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        for (auto& e : mComputeDone) INFMOE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        INFMOE_HIP(hipEventCreateWithFlags(&mFork, hipEventDisableTiming));
+    }
+    mInitialized = true;
+    if (!mScoreBias.empty()) INFMOE_TRY(setScoreBias(mScoreBias.data()));
+    return INFMOE_OK;
+}
+
+Status MoELayer::terminate() {
+    // plugin/MoELayerPlugin.cc:203-237.  The sub-layer is shared with clones and releases its
+    // weights when its last owner goes away.
+    if (mCentroidsGpu) (void)hipFree(mCentroidsGpu);
+    if (mLayernormGpu) (void)hipFree(mLayernormGpu);
+    if (mScoreBiasGpu) (void)hipFree(mScoreBiasGpu);
+    if (mRoutingGpu) (void)hipFree(mRoutingGpu);
+    if (mRoutingHost) (void)hipHostFree(mRoutingHost);
+    mCentroidsGpu = mLayernormGpu = mScoreBiasGpu = nullptr;
+    mRoutingGpu = mRoutingHost = nullptr;
+    if (mCopyStream) (void)hipStreamDestroy(mCopyStream);
+    mCopyStream = nullptr;
+    for (auto s : mComputeStreams) (void)hipStreamDestroy(s);
+    mComputeStreams.clear();
+    for (auto* v : {&mCopyDone, &mComputeDone, &mJoin}) {
+        for (auto e : *v) (void)hipEventDestroy(e);
+        v->clear();
+    }
+    if (mFork) (void)hipEventDestroy(mFork);
+    if (mRoutingDone) (void)hipEventDestroy(mRoutingDone);
+    mFork = mRoutingDone = nullptr;
+    mInitialized = false;
+    return INFMOE_OK;
+}
+
+// ---------------------------------------------------------------- enqueue
+
+Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const* inputs, void* const* outputs,
+                         void* workspace, hipStream_t stream) {
+    int T = 0;
+    INFMOE_TRY(checkDims(dims, nbDims, &T));
+    if (!mInitialized) return fail(INFMOE_ERR_STATE, "enqueue before initialize");
+    if (inputs == nullptr || outputs == nullptr || inputs[0] == nullptr || outputs[0] == nullptr)
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "null input or output");
+    if (T == 0) return INFMOE_OK;
+    if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255))
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "workspace must be non-null and 256-byte aligned");
+    const int E = mParams.expertCount, d = mParams.embeddingSize;
+    const float* x = static_cast<const float*>(inputs[0]);
+    float* y = static_cast<float*>(outputs[0]);
+    Carve c;
+    INFMOE_TRY(carve(T, workspace, &c));
+    int32_t* dCount = mRoutingGpu;
+    int32_t* dOffset = dCount + E;
+    int32_t* dStats = dOffset + E + 1;
+    mSublayer->setLayerTokenCount(T);
+
+    // 0-2. norm (cpm_2: for scoring only), scores, top-1          plugin/MoELayerPlugin.cc:312-345
+    INFMOE_HIP(launch_fill_i32(dStats, 4, 0, stream));
+    const bool ln = mParams.flags.layernormOnInputBeforeScore;
+    INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
+                                mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream));
+    // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
+    const bool grouped = resident();
+    const int skinnyMax = grouped ? mSublayer->skinnyMaxRows(T) : 0;
+    INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, grouped ? c.tiles : nullptr,
+                                   grouped ? c.nTiles : nullptr, kGemmTileRows, skinnyMax, c.rowExpert, stream));
+    INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream));  // experts see the raw input (:354)
+    INFMOE_HIP(hipEventRecord(mRoutingDone, stream));
+
+    // 4. experts                                                   plugin/MoELayerPlugin.cc:360-402
+    if (grouped) {
+        GroupedRun g;
+        g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
+        g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
+        g.tiles = c.tiles, g.nTiles = c.nTiles, g.maxTiles = c.maxTiles, g.stream = stream;
+        INFMOE_TRY(mSublayer->runGrouped(g));
+    } else {
+        INFMOE_TRY(runStreamed(T, c, stream));
+    }
+
+    // 6-7. mix (base_layer) and un-shuffle                         plugin/MoELayerPlugin.cc:404-412
+    // (the post-expert rows are gathered; :411 of the public reference passes the pre-expert ones)
+    if (mParams.flags.baseLayerOutputMix)
+        INFMOE_HIP(launch_mix_gather(T, d, c.pos, c.routed, c.post, c.routedCoeff, y, stream));
+    else
+        INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream));
+    return INFMOE_OK;
+}
+
+// Experts streamed through max_concurrency device slots (plugin/MoELayerPlugin.cc:360-402).
+// The host learns the token counts once (one blocking copy of E integers), then queues every
+// copy and every expert without blocking again:
+//   copy stream:   [wait: expert k-mc done] copy expert k into slot k % mc, signal copyDone[k]
+//   compute k%n:   [wait: copyDone[k]] run expert k from its slot,          signal computeDone[k]
+// so up to mc-1 experts are prefetched while one computes (the reference prefetches one), and
+// max_concurrency = 1 degenerates to copy, compute, copy, ... with no overlap.
+Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
+    const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
+    const size_t routingInts = (size_t)2 * E + 1 + 4;
+    INFMOE_HIP(hipMemcpyAsync(mRoutingHost, mRoutingGpu, sizeof(int32_t) * routingInts, hipMemcpyDeviceToHost, stream));
+    INFMOE_HIP(hipStreamSynchronize(stream));
+    const int32_t* count = mRoutingHost;
+    const int32_t* offset = mRoutingHost + E;
+    const int32_t* stats = offset + E + 1;
+    if (stats[1] > 0) return fail(INFMOE_ERR_NAN, "%d token(s) have no orderable score (NaN input?)", stats[1]);
+
+    INFMOE_HIP(hipEventRecord(mFork, stream));
+    INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
+    for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
+    int k = 0;
+    for (int e = 0; e < E; ++e) {  // ascending, empty experts skipped (:361-363,383-384)
+        if (count[e] == 0) continue;
+        const int slot = k % mc;
+        char* slotPtr = c.slots + c.slotStride * (size_t)slot;
+        if (k >= mc) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[k - mc], 0));
+        INFMOE_TRY(mSublayer->copyWeights(slotPtr, e, mCopyStream));
+        INFMOE_HIP(hipEventRecord(mCopyDone[k], mCopyStream));
+        hipStream_t cs = mComputeStreams[k % mComputeStreams.size()];
+        INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
+        // rows of different experts are disjoint, so each expert gets its own stretch of the
+        // shared scratch (row stride applied: the public reference omits it at :373,391-392)
+        INFMOE_TRY(mSublayer->run(count[e], slotPtr, c.routed + (size_t)offset[e] * d, c.post + (size_t)offset[e] * d,
+                                  c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
+        INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
+        ++k;
+    }
+    for (size_t i = 0; i < mComputeStreams.size(); ++i) {
+        INFMOE_HIP(hipEventRecord(mJoin[i], mComputeStreams[i]));
+        INFMOE_HIP(hipStreamWaitEvent(stream, mJoin[i], 0));
+    }
+    return INFMOE_OK;
+}
+
+Status MoELayer::lastRouting(int32_t* countHost, int32_t* statsHost) {
+    if (!mInitialized) return fail(INFMOE_ERR_STATE, "no routing before initialize");
+    const int E = mParams.expertCount;
+    INFMOE_HIP(hipEventSynchronize(mRoutingDone));
+    std::vector<int32_t> tmp((size_t)2 * E + 1 + 4);
+    INFMOE_HIP(hipMemcpy(tmp.data(), mRoutingGpu, sizeof(int32_t) * tmp.size(), hipMemcpyDeviceToHost));
+    if (countHost) memcpy(countHost, tmp.data(), sizeof(int32_t) * E);
+    if (statsHost) memcpy(statsHost, tmp.data() + 2 * E + 1, sizeof(int32_t) * 3);
+    return INFMOE_OK;
+}
+
+// ---------------------------------------------------------------- serialisation
+// Own little-endian format (the reference's has known defects, plugin/MoELayerPlugin.cc:131-140,
+// 418-423,451-453, and is not reproduced):
+//   u32 magic 'IMOE', u32 version = 1,
+//   i32 E, d, h, mc, normKind, ffnKind, u32 flags (bit0 norm-before-score, bit1 base-layer mix),
+//   u32 len(weight_file), len(sublayer_type), len(variant), n_centroids, n_layernorm,
+//   the three strings (no terminator), zero padding to a multiple of 4, centroids, layernorm.
+namespace {
+constexpr uint32_t kMagic = 0x454F4D49u, kVersion = 1u;
+constexpr size_t kHeaderWords = 14;
+}
+
+Status MoELayer::serializationSize(size_t* bytes) const {
+    const size_t strings = mParams.weightFile.size() + mParams.sublayerType.size() + mParams.variant.size();
+    *bytes = kHeaderWords * 4 + align_up(strings, 4) + 4 * (mParams.centroids.size() + mParams.layernormWeight.size());
+    return INFMOE_OK;
+}
+
+Status MoELayer::serialize(void* buffer, size_t bytes) const {
+    size_t need = 0;
+    serializationSize(&need);
+    if (buffer == nullptr || bytes < need) return fail(INFMOE_ERR_INVALID_ARGUMENT, "serialize needs %zu bytes", need);
+    memset(buffer, 0, need);
+    uint32_t* w = static_cast<uint32_t*>(buffer);
+    const uint32_t head[kHeaderWords] = {kMagic, kVersion, (uint32_t)mParams.expertCount, (uint32_t)mParams.embeddingSize,
+                                         (uint32_t)mParams.hiddenSize, (uint32_t)mParams.maxConcurrency, (uint32_t)mParams.normKind,
+                                         (uint32_t)mParams.ffnKind,
+                                         (mParams.flags.layernormOnInputBeforeScore ? 1u : 0u) | (mParams.flags.baseLayerOutputMix ? 2u : 0u),
+                                         (uint32_t)mParams.weightFile.size(), (uint32_t)mParams.sublayerType.size(),
+                                         (uint32_t)mParams.variant.size(), (uint32_t)mParams.centroids.size(),
+                                         (uint32_t)mParams.layernormWeight.size()};
+    memcpy(w, head, sizeof(head));
+    char* p = static_cast<char*>(buffer) + sizeof(head);
+    char* s = p;
+    for (const std::string* str : {&mParams.weightFile, &mParams.sublayerType, &mParams.variant}) {
+        memcpy(s, str->data(), str->size());
+        s += str->size();
+    }
+    p += align_up((size_t)(s - p), 4);
+    memcpy(p, mParams.centroids.data(), 4 * mParams.centroids.size());
+    p += 4 * mParams.centroids.size();
+    memcpy(p, mParams.layernormWeight.data(), 4 * mParams.layernormWeight.size());
+    return INFMOE_OK;
+}
+
+Status MoELayer::deserialize(const char* layerName, const void* data, size_t bytes, std::unique_ptr<MoELayer>* out) {
+    if (data == nullptr || bytes < kHeaderWords * 4) return fail(INFMOE_ERR_INVALID_ARGUMENT, "serialized layer is truncated");
+    uint32_t head[kHeaderWords];
+    memcpy(head, data, sizeof(head));
+    if (head[0] != kMagic || head[1] != kVersion) return fail(INFMOE_ERR_INVALID_ARGUMENT, "not a serialized MoE layer of this version");
+    MoEParams p;
+    p.layerName = layerName ? layerName : "";
+    p.expertCount = (int)head[2], p.embeddingSize = (int)head[3], p.hiddenSize = (int)head[4], p.maxConcurrency = (int)head[5];
+    p.normKind = (int)head[6], p.ffnKind = (int)head[7];
+    const size_t l1 = head[9], l2 = head[10], l3 = head[11], nc = head[12], nl = head[13];
+    const size_t need = sizeof(head) + align_up(l1 + l2 + l3, 4) + 4 * (nc + nl);
+    if (bytes < need) return fail(INFMOE_ERR_INVALID_ARGUMENT, "serialized layer is truncated: %zu of %zu bytes", bytes, need);
+    const char* s = static_cast<const char*>(data) + sizeof(head);
+    p.weightFile.assign(s, l1);
+    p.sublayerType.assign(s + l1, l2);
+    p.variant.assign(s + l1 + l2, l3);
+    const char* f = s + align_up(l1 + l2 + l3, 4);
+    p.centroids.resize(nc);
+    memcpy(p.centroids.data(), f, 4 * nc);
+    p.layernormWeight.resize(nl);
+    memcpy(p.layernormWeight.data(), f + 4 * nc, 4 * nl);
+    return create(std::move(p), out);
+}
+
+}  // namespace infmoe

@@ -1,0 +1,222 @@
+#include "t5ff_layer.h"
+
+#include <cstring>
+
+#include "../npz_reader.h"
+#include "identity_layer.h"
+
+namespace infmoe {
+
+T5FFLayer::T5FFLayer(int expertCount, int embeddingSize, int hiddenSize, const char* weightFile, int maxConcurrency,
+                     int normKind, int ffnKind)
+    : MoESubLayer(expertCount, embeddingSize, hiddenSize, weightFile, maxConcurrency),
+      mNormKind(normKind),
+      mFfnKind(ffnKind) {}
+
+T5FFLayer::~T5FFLayer() { terminate(); }
+
+bool T5FFLayer::configureWithFormat(const Dims* in, int32_t nbInputs, const Dims* out, int32_t nbOutputs) {
+    // plugin/sublayers/T5FFLayer.cc:20-36
+    if (nbInputs != 1 || nbOutputs != 1) return false;
+    if (in[0].nbDims != 3 || out[0].nbDims != 3) return false;
+    for (int i = 0; i < 3; ++i)
+        if (in[0].d[i] != out[0].d[i]) return false;
+    return in[0].d[2] == mEmbeddingSize;
+}
+
+size_t T5FFLayer::weightBytes(int d, int h, int ffnKind) {
+    const size_t mats = ffnKind == FFN_GATED_GELU ? 3 : 2;
+    return sizeof(float) * ((size_t)d + mats * (size_t)d * (size_t)h);  // plugin/sublayers/T5FFLayer.cc:43
+}
+
+size_t T5FFLayer::workspaceBytes(int rows, int d, int h) {
+    return sizeof(float) * (size_t)rows * ((size_t)d + (size_t)h);
+}
+
+size_t T5FFLayer::weightSize() { return weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind); }
+
+size_t T5FFLayer::workspaceSize(int32_t tokenCount) {
+    return align_up(workspaceBytes(tokenCount, mEmbeddingSize, mHiddenSize));
+}
+
+int T5FFLayer::keyIndex(const char* key, size_t* off, size_t* cnt) const {
+    const size_t d = mEmbeddingSize, dh = (size_t)mEmbeddingSize * mHiddenSize;
+    if (strcmp(key, "layer_norm_weight") == 0) {
+        *off = 0, *cnt = d;
+        return 0;
+    }
+    if (mFfnKind == FFN_GATED_GELU) {
+        if (strcmp(key, "wi_0_weight") == 0) return *off = d, *cnt = dh, 1;
+        if (strcmp(key, "wi_1_weight") == 0) return *off = d + dh, *cnt = dh, 2;
+        if (strcmp(key, "wo_weight") == 0) return *off = d + 2 * dh, *cnt = dh, 3;
+    } else {
+        if (strcmp(key, "wi_weight") == 0) return *off = d, *cnt = dh, 1;
+        if (strcmp(key, "wo_weight") == 0) return *off = d + dh, *cnt = dh, 2;
+    }
+    return -1;
+}
+
+Status T5FFLayer::ensureHostStore() {
+    if (mHostWeights != nullptr) return INFMOE_OK;
+    // page-locked like the reference's npz store (plugin/thirdparty/cnpy/cnpy.h:27-39), so that
+    // hipMemcpyAsync from it really is asynchronous
+    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mHostWeights), slotStride() * (size_t)mExpertCount,
+                             hipHostMallocDefault));
+    mHave.assign((size_t)mExpertCount * (nMatrices() + 1), 0);
+    return INFMOE_OK;
+}
+
+Status T5FFLayer::setWeights(int expert, const char* key, const float* host, size_t count) {
+    if (expert < 0 || expert >= mExpertCount) return fail(INFMOE_ERR_INVALID_ARGUMENT, "expert %d out of range", expert);
+    if (key == nullptr || host == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null key or data");
+    size_t off = 0, cnt = 0;
+    const int idx = keyIndex(key, &off, &cnt);
+    if (idx < 0) return fail(INFMOE_ERR_UNKNOWN_FIELD, "unknown weight key for this ffn kind: %s", key);
+    // the reference asserts on the byte count of every array (plugin/sublayers/T5FFLayer.cc:62,69,76,83)
+    if (count != cnt) return fail(INFMOE_ERR_INVALID_ARGUMENT, "%s: expected %zu floats, got %zu", key, cnt, count);
+    INFMOE_TRY(ensureHostStore());
+    float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)expert);
+    memcpy(slot + off, host, cnt * sizeof(float));
+    mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
+    return INFMOE_OK;
+}
+
+Status T5FFLayer::initialize() {
+    // plugin/sublayers/T5FFLayer.cc:143-147
+    if (mHostWeights == nullptr) {
+        if (mWeightFile.empty()) return fail(INFMOE_ERR_STATE, "T5_FF: no expert_weight_file and no weights given by pointer");
+        NpzReader npz;
+        INFMOE_TRY(npz.open(mWeightFile.c_str()));
+        INFMOE_TRY(ensureHostStore());
+        static const char* kGated[] = {"layer_norm_weight", "wi_0_weight", "wi_1_weight", "wo_weight"};
+        static const char* kRelu[] = {"layer_norm_weight", "wi_weight", "wo_weight"};
+        const char* const* keys = mFfnKind == FFN_GATED_GELU ? kGated : kRelu;
+        for (int e = 0; e < mExpertCount; ++e) {
+            float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)e);
+            for (int j = 0; j <= nMatrices(); ++j) {
+                size_t off = 0, cnt = 0;
+                keyIndex(keys[j], &off, &cnt);
+                const std::string name = std::to_string(e) + "/" + keys[j];  // README.md:121
+                INFMOE_TRY(npz.read_f32(name.c_str(), slot + off, cnt));
+                mHave[(size_t)e * (nMatrices() + 1) + j] = 1;
+            }
+        }
+    }
+    for (size_t i = 0; i < mHave.size(); ++i)
+        if (!mHave[i])
+            return fail(INFMOE_ERR_MISSING_FIELD, "T5_FF: expert %zu is missing weight array #%zu", i / (nMatrices() + 1),
+                        i % (nMatrices() + 1));
+    return INFMOE_OK;
+}
+
+void T5FFLayer::terminate() {
+    // plugin/sublayers/T5FFLayer.cc:149-156
+    if (mDeviceWeights) (void)hipFree(mDeviceWeights);
+    mDeviceWeights = nullptr;
+    if (mHostWeights) (void)hipHostFree(mHostWeights);
+    mHostWeights = nullptr;
+    mHave.clear();
+}
+
+Status T5FFLayer::makeResident() {
+    if (mDeviceWeights != nullptr) return INFMOE_OK;
+    if (mHostWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: makeResident before initialize");
+    const size_t bytes = slotStride() * (size_t)mExpertCount;
+    INFMOE_HIP(hipMalloc(&mDeviceWeights, bytes));
+    INFMOE_HIP(hipMemcpy(mDeviceWeights, mHostWeights, bytes, hipMemcpyHostToDevice));
+    return INFMOE_OK;
+}
+
+Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
+    // plugin/sublayers/T5FFLayer.cc:55-88 issues four copies; the host store is already packed in
+    // slot order, so one copy moves the expert.
+    if (mHostWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: copyWeights before initialize");
+    const char* src = reinterpret_cast<const char*>(mHostWeights) + slotStride() * (size_t)expert;
+    INFMOE_HIP(hipMemcpyAsync(dst, src, weightSize(), hipMemcpyHostToDevice, stream));
+    return INFMOE_OK;
+}
+
+// Few-row kernels are used for an expert only when the whole call is decode-like, and the rule
+// depends on nothing but (tokens of the call, experts, rows of the expert), so that the grouped
+// and the per-expert schedules pick the same kernel for the same expert and agree bit for bit.
+static bool decode_like(int layerTokens, int expertCount) { return layerTokens <= 16 * expertCount; }
+
+int T5FFLayer::skinnyMaxRows(int32_t tokenCount) const {
+    return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kSkinnyMaxRows : 0;
+}
+
+Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int h, int normKind, int ffnKind,
+                         const void* weights, const float* in, float* out, void* workspace, hipStream_t stream) {
+    if (rows <= 0) return INFMOE_OK;
+    const float* w = static_cast<const float*>(weights);
+    const size_t dh = (size_t)d * h;
+    float* ln = static_cast<float*>(workspace);
+    float* hid = ln + (size_t)rows * d;
+    // plugin/sublayers/T5FFLayer.cc:99-103
+    INFMOE_HIP(launch_row_norm(ln, in, rows, d, w, 0, nullptr, normKind, stream));
+    GemmProblem g1{};  // plugin/sublayers/T5FFLayer.cc:112-126
+    g1.A = ln, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
+    g1.B1 = ffnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
+    g1.epilogue = ffnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
+    GemmProblem g2{};  // plugin/sublayers/T5FFLayer.cc:130-138 (residual instead of copy + beta = 1)
+    g2.A = hid, g2.B = w + d + (ffnKind == FFN_GATED_GELU ? 2 : 1) * dh, g2.R = in, g2.C = out, g2.N = d, g2.K = h;
+    g2.epilogue = EPI_RESIDUAL;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(ln)) & 15) == 0;
+    const bool skinny = rows <= kSkinnyMaxRows && decode_like(layerTokens, expertCount) && d % 4 == 0 && h % 4 == 0 && aligned;
+    if (skinny) {
+        INFMOE_HIP(launch_expert_skinny(g1, rows, stream));
+        INFMOE_HIP(launch_expert_skinny(g2, rows, stream));
+    } else {
+        INFMOE_HIP(launch_expert_gemm(g1, rows, stream));
+        INFMOE_HIP(launch_expert_gemm(g2, rows, stream));
+    }
+    return INFMOE_OK;
+}
+
+Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
+                      hipStream_t stream) {
+    // outside a layer call (token count of the call unknown) the expert stands alone
+    const bool inLayer = mLayerTokenCount > 0;
+    return runOne(tokenCount, inLayer ? mLayerTokenCount : tokenCount, inLayer ? mExpertCount : 1,
+                  mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights, static_cast<const float*>(input),
+                  static_cast<float*>(output), workspace, stream);
+}
+
+Status T5FFLayer::runGrouped(const GroupedRun& g) {
+    if (mDeviceWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: runGrouped needs resident weights");
+    const int T = g.tokenCount, d = mEmbeddingSize, h = mHiddenSize;
+    const size_t dh = (size_t)d * h, stride = slotStride() / sizeof(float);
+    const float* w = static_cast<const float*>(mDeviceWeights);
+    float* ln = static_cast<float*>(g.workspace);
+    float* hid = ln + (size_t)T * d;
+    INFMOE_HIP(launch_row_norm(ln, g.input, T, d, w, stride, g.rowExpert, mNormKind, g.stream));
+    GemmProblem g1{};
+    g1.A = ln, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
+    g1.B1 = mFfnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
+    g1.epilogue = mFfnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
+    GemmProblem g2{};
+    g2.A = hid, g2.B = w + d + (mFfnKind == FFN_GATED_GELU ? 2 : 1) * dh, g2.R = g.input, g2.C = g.output, g2.N = d, g2.K = h;
+    g2.epilogue = EPI_RESIDUAL;
+    const bool skinny = skinnyMaxRows(T) > 0;
+    INFMOE_HIP(launch_expert_gemm_grouped(g1, stride, g.tiles, g.nTiles, g.maxTiles, g.stream));
+    if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g1, stride, g.count, g.offset, mExpertCount, g.stream));
+    INFMOE_HIP(launch_expert_gemm_grouped(g2, stride, g.tiles, g.nTiles, g.maxTiles, g.stream));
+    if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g2, stride, g.count, g.offset, mExpertCount, g.stream));
+    return INFMOE_OK;
+}
+
+Status make_sublayer(const char* type, int expertCount, int embeddingSize, int hiddenSize, const char* weightFile,
+                     int maxConcurrency, int normKind, int ffnKind, std::shared_ptr<MoESubLayer>* out) {
+    // plugin/MoELayerPlugin.cc:28-41, names from plugin/MoELayerPlugin.h:23-26
+    if (type != nullptr && strcmp(type, "T5_FF") == 0) {
+        *out = std::make_shared<T5FFLayer>(expertCount, embeddingSize, hiddenSize, weightFile, maxConcurrency, normKind, ffnKind);
+        return INFMOE_OK;
+    }
+    if (type != nullptr && strcmp(type, "Identity") == 0) {
+        *out = std::make_shared<IdentityLayer>();
+        return INFMOE_OK;
+    }
+    return fail(INFMOE_ERR_UNSUPPORTED, "unsupported sublayer type: %s", type ? type : "(null)");
+}
+
+}  // namespace infmoe

@@ -1,0 +1,212 @@
+"""Parity of every kernel-level C entry point against the float64 oracle, on the GPU."""
+import numpy as np
+import pytest
+
+from infmoe_amd import capi
+from oracle import moe_oracle as O
+from tests.gpu_util import assert_close, check_assignment, dev, pack_slot, stream_ptr
+
+pytestmark = pytest.mark.gpu
+NORM = capi.NORM_KINDS
+FFN = capi.FFN_KINDS
+
+
+# ------------------------------------------------------------------ gating
+def run_gate(lib, torch, x, c, gamma, norm, bias=None):
+    T, d = x.shape
+    E = c.shape[0]
+    dx, dc = dev(torch, x), dev(torch, c)
+    dg = dev(torch, gamma) if gamma is not None else None
+    db = dev(torch, bias) if bias is not None else None
+    sel = torch.full((T,), -7, dtype=torch.int32, device="cuda")
+    coeff = torch.zeros(T, dtype=torch.float32, device="cuda")
+    stats = torch.zeros(4, dtype=torch.int32, device="cuda")
+    capi.check(lib.infmoe_gate_top1(T, d, E, dx.data_ptr(), dc.data_ptr(), dg.data_ptr() if dg is not None else None,
+                                    NORM[norm], db.data_ptr() if db is not None else None, sel.data_ptr(),
+                                    coeff.data_ptr(), stats.data_ptr(), stream_ptr(torch)))
+    torch.cuda.synchronize()
+    return sel.cpu().numpy(), coeff.cpu().numpy(), stats.cpu().numpy()
+
+
+@pytest.mark.parametrize("T,d,E,norm,use_bias", [
+    (32, 64, 4, "none", False),      # tiny default-variant config
+    (80, 4, 2, "rms", False),        # reference example shape (d smaller than one chunk)
+    (100, 4096, 32, "rms", False),   # cpm_2 shape
+    (77, 130, 5, "centered", False), # row length not a multiple of 4: scalar path
+    (1, 256, 16, "rms", False),
+    (300, 2048, 64, "none", True),   # base_layer shape with score bias
+    (50, 512, 200, "centered", True),  # more than 128 experts: several passes
+    (64, 4096, 32, "centered", False),
+])
+def test_gate_top1_matches_oracle(lib, torch_cuda, T, d, E, norm, use_bias):
+    torch = torch_cuda
+    x, c, g = O.draw_inputs(11, T, d, E)
+    x = x + (0.3 if norm == "centered" else 0.0)  # a mean for the centred norm to remove
+    bias = (0.2 * np.random.default_rng(5).standard_normal(E)).astype(np.float32) if use_bias else None
+    sel, coeff, stats = run_gate(lib, torch, x, c, g if norm != "none" else None, norm, bias)
+    xa = O.layernorm(x, g, norm) if norm != "none" else x.astype(np.float64)
+    aff = O.score(xa, c, bias)
+    exempt = check_assignment(sel, aff)
+    assert stats[0] == exempt
+    assert stats[1] == 0
+    want = aff[np.arange(T), sel]
+    assert_close(coeff, want, what="coeff")
+
+
+def test_gate_top1_exact_ties_pick_lowest_index(lib, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    T, d, E = 64, 32, 24
+    x = rng.integers(-2, 3, size=(T, d)).astype(np.float32)  # small integers: scores are exact
+    c = rng.integers(-1, 2, size=(E, d)).astype(np.float32)
+    c[7] = c[3]
+    c[19] = c[3]  # identical centroids -> exact ties
+    sel, coeff, stats = run_gate(lib, torch, x, c, None, "none")
+    aff = O.score(x, c)
+    want, best = O.select_top1(aff)
+    np.testing.assert_array_equal(sel, want)  # lowest index among equal maxima, also after re-scoring
+    np.testing.assert_array_equal(coeff, best.astype(np.float32))
+    assert stats[0] == int((O.top2_relative_gap(aff) < 1e-6).sum())
+
+
+def test_gate_top1_counts_nan_rows(lib, torch_cuda):
+    torch = torch_cuda
+    x, c, g = O.draw_inputs(2, 40, 64, 8)
+    x[5, 3] = np.nan
+    x[33, :] = np.nan
+    sel, coeff, stats = run_gate(lib, torch, x, c, g, "rms")
+    assert stats[1] == 2
+    ok = np.ones(40, bool)
+    ok[[5, 33]] = False
+    aff = O.score(O.layernorm(x[ok], g, "rms"), c)
+    np.testing.assert_array_equal(sel[ok], O.select_top1(aff)[0])
+
+
+def test_gate_near_tie_is_rescored_in_float64(lib, torch_cuda):
+    """Two centroids 3e-6 relative apart: above the 1e-6 exemption, at the edge of what FP32
+    accumulation over 1024 terms can order, so the float64 re-scoring has to decide."""
+    torch = torch_cuda
+    T, d, E = 48, 1024, 8
+    x, c, g = O.draw_inputs(4, T, d, E)
+    c = c.astype(np.float64)
+    c[:] *= 0.1
+    c[5] = 1.0 * np.sign(np.arange(d) % 2 - 0.5) / np.sqrt(d)
+    c = c.astype(np.float32)
+    c[2] = (c[5].astype(np.float64) * (1 + 3e-6)).astype(np.float32)  # 3e-6 relative apart: must be ordered
+    sel, coeff, stats = run_gate(lib, torch, x, c, None, "none")
+    aff = O.score(x, c)
+    exempt = check_assignment(sel, aff)
+    assert stats[2] >= 1  # the float64 path ran
+    assert stats[0] == exempt
+
+
+# ------------------------------------------------------------------ count / sort
+@pytest.mark.parametrize("T,E,mode", [
+    (1, 1, "rand"), (1, 4, "rand"), (32, 4, "rand"), (1023, 7, "rand"), (1024, 32, "rand"), (1025, 32, "rand"),
+    (4096, 32, "rand"), (16384, 64, "zipf"), (5000, 300, "rand"), (3000, 5, "one"),
+])
+def test_expert_count_is_bit_exact(lib, torch_cuda, T, E, mode):
+    torch = torch_cuda
+    rng = np.random.default_rng(T * 31 + E)
+    if mode == "rand":
+        sel = rng.integers(0, E, size=T).astype(np.int32)
+    elif mode == "one":
+        sel = np.full(T, E - 2, np.int32)
+    else:
+        p = np.arange(1, E + 1) ** -1.2
+        sel = rng.choice(E, size=T, p=p / p.sum()).astype(np.int32)
+    dsel = dev(torch, sel)
+    pos = torch.full((T,), -1, dtype=torch.int32, device="cuda")
+    count = torch.full((E,), -1, dtype=torch.int32, device="cuda")
+    offset = torch.full((E + 1,), -1, dtype=torch.int32, device="cuda")
+    scratch = torch.empty(max(lib.infmoe_expert_count_scratch_bytes(T, E), 1), dtype=torch.uint8, device="cuda")
+    capi.check(lib.infmoe_expert_count(T, E, dsel.data_ptr(), pos.data_ptr(), count.data_ptr(), offset.data_ptr(),
+                                       scratch.data_ptr(), stream_ptr(torch)))
+    torch.cuda.synchronize()
+    wc, wo, wp = O.expert_count(sel, E)
+    np.testing.assert_array_equal(count.cpu().numpy(), wc)
+    np.testing.assert_array_equal(offset.cpu().numpy(), wo)
+    np.testing.assert_array_equal(pos.cpu().numpy(), wp)
+
+
+# ------------------------------------------------------------------ scatter / gather / mix
+@pytest.mark.parametrize("T,d", [(1, 4), (33, 64), (257, 130), (512, 4096), (100, 2048)])
+def test_scatter_gather_mix(lib, torch_cuda, T, d):
+    torch = torch_cuda
+    rng = np.random.default_rng(T + d)
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    coeff = rng.standard_normal(T).astype(np.float32)
+    pos = rng.permutation(T).astype(np.int32)
+    dx, dc, dp = dev(torch, x), dev(torch, coeff), dev(torch, pos)
+    routed = torch.zeros_like(dx)
+    rc = torch.zeros_like(dc)
+    s = stream_ptr(torch)
+    capi.check(lib.infmoe_expert_scatter(T, d, dx.data_ptr(), dc.data_ptr(), dp.data_ptr(), routed.data_ptr(), rc.data_ptr(), s))
+    wr, wrc = O.scatter(x, coeff, pos)
+    np.testing.assert_array_equal(routed.cpu().numpy(), wr)
+    np.testing.assert_array_equal(rc.cpu().numpy(), wrc)
+    back = torch.zeros_like(dx)
+    capi.check(lib.infmoe_expert_gather(T, d, routed.data_ptr(), dp.data_ptr(), back.data_ptr(), s))
+    np.testing.assert_array_equal(back.cpu().numpy(), x)  # gather(scatter(x)) == x exactly
+    post = rng.standard_normal((T, d)).astype(np.float32)
+    dpost = dev(torch, post)
+    out = torch.zeros_like(dx)
+    capi.check(lib.infmoe_expert_mix_gather(T, d, dp.data_ptr(), routed.data_ptr(), dpost.data_ptr(), rc.data_ptr(), out.data_ptr(), s))
+    want = O.mix_and_gather(post, wr, wrc, pos)
+    assert_close(out.cpu().numpy(), want, rtol=1e-6, what="mix")
+
+
+# ------------------------------------------------------------------ norm
+@pytest.mark.parametrize("rows,d", [(1, 4), (5, 64), (37, 130), (64, 4096), (3, 10240), (2, 8200)])
+@pytest.mark.parametrize("kind", ["rms", "centered"])
+def test_layernorm(lib, torch_cuda, rows, d, kind):
+    torch = torch_cuda
+    rng = np.random.default_rng(rows * 7 + d)
+    x = (rng.standard_normal((rows, d)) * 2 + 0.7).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    dx, dg = dev(torch, x), dev(torch, g)
+    out = torch.zeros_like(dx)
+    capi.check(lib.infmoe_layernorm(out.data_ptr(), dx.data_ptr(), rows, d, dg.data_ptr(), NORM[kind], stream_ptr(torch)))
+    assert_close(out.cpu().numpy(), O.layernorm(x, g, kind), rtol=1e-5, what="norm")
+
+
+# ------------------------------------------------------------------ expert
+def run_t5ff(lib, torch, x, w, norm, ffn):
+    rows, d = x.shape
+    h = w["wo_weight"].shape[1]
+    slot = dev(torch, pack_slot(w, ffn))
+    assert slot.numel() * 4 == lib.infmoe_t5ff_weight_bytes(d, h, FFN[ffn])
+    dx = dev(torch, x)
+    out = torch.zeros_like(dx)
+    ws = torch.empty(max(lib.infmoe_t5ff_workspace_bytes(rows, d, h, FFN[ffn]), 16), dtype=torch.uint8, device="cuda")
+    capi.check(lib.infmoe_t5ff_run(rows, d, h, NORM[norm], FFN[ffn], slot.data_ptr(), dx.data_ptr(), out.data_ptr(),
+                                   ws.data_ptr(), stream_ptr(torch)))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 8, 9, 16, 17, 100, 128, 140, 255, 256, 257, 300, 600])
+def test_t5ff_row_counts(lib, torch_cuda, rows):
+    d, h = 64, 256
+    w = O.draw_expert(21, 0, d, h, "relu")
+    x = O.draw_inputs(rows, rows, d, 2)[0]
+    got = run_t5ff(lib, torch_cuda, x, w, "rms", "relu")
+    assert_close(got, O.t5ff_run(x, w, "rms", "relu"), what=f"t5ff rows={rows}")
+
+
+@pytest.mark.parametrize("d,h", [(64, 256), (128, 320), (20, 36), (6, 10), (512, 1280), (4096, 256)])
+@pytest.mark.parametrize("norm,ffn", [("rms", "relu"), ("centered", "gated_gelu"), ("rms", "gated_gelu"), ("centered", "relu")])
+@pytest.mark.parametrize("rows", [4, 70])
+def test_t5ff_shapes_and_kinds(lib, torch_cuda, d, h, norm, ffn, rows):
+    w = O.draw_expert(22, 1, d, h, ffn)
+    x = O.draw_inputs(5, rows, d, 2)[0] + 0.25
+    got = run_t5ff(lib, torch_cuda, x, w, norm, ffn)
+    assert_close(got, O.t5ff_run(x, w, norm, ffn), what=f"t5ff {d}x{h} {norm} {ffn}")
+
+
+def test_t5ff_zero_wo_returns_input(lib, torch_cuda):
+    d, h = 64, 128
+    w = O.draw_expert(23, 0, d, h, "relu")
+    w["wo_weight"][:] = 0
+    x = O.draw_inputs(6, 40, d, 2)[0]
+    np.testing.assert_array_equal(run_t5ff(lib, torch_cuda, x, w, "rms", "relu"), x)
