@@ -135,6 +135,19 @@ void infmoe_destroy(infmoe_plugin* p);
  */
 int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stats_host);
 
+/*
+ * Phase timing (no counterpart in the reference, which only prints wall time from Python,
+ * python/examples/stacked_moe.py:55-60).  When enabled, infmoe_enqueue records HIP events on its
+ * stream at the phase boundaries; infmoe_last_timing waits for the last call and returns the
+ * elapsed milliseconds of: [0] gating, [1] count+sort, [2] scatter, [3] expert norm,
+ * [4] first expert GEMM (activation fused), [5] second expert GEMM (residual fused),
+ * [6] gather / mix.  Phases 3-5 are only separated when all experts are resident (otherwise the
+ * whole streamed expert loop is reported in [4]).  `ms` holds INFMOE_N_PHASES floats.
+ */
+#define INFMOE_N_PHASES 7
+int32_t infmoe_set_timing(infmoe_plugin* p, int32_t enable);
+int32_t infmoe_last_timing(infmoe_plugin* p, float* ms);
+
 /* Replaces getSerializationSize / serialize / deserializePlugin (plugin/MoELayerPlugin.cc:104-143,418-458).
  * A versioned little-endian format of this library's own; expert weights are not serialised,
  * only the file path, as in the reference. */

@@ -47,6 +47,8 @@ PROTOTYPES = {
     "infmoe_terminate": (_i32, [_vp]),
     "infmoe_destroy": (None, [_vp]),
     "infmoe_last_routing": (_i32, [_vp, _pi32, _pi32]),
+    "infmoe_set_timing": (_i32, [_vp, _i32]),
+    "infmoe_last_timing": (_i32, [_vp, C.POINTER(C.c_float)]),
     "infmoe_serialization_size": (_i32, [_vp, C.POINTER(_sz)]),
     "infmoe_serialize": (_i32, [_vp, _vp, _sz]),
     "infmoe_deserialize": (_i32, [C.c_char_p, _vp, _sz, C.POINTER(_vp)]),

@@ -185,6 +185,21 @@ int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stat
     });
 }
 
+int32_t infmoe_set_timing(infmoe_plugin* p, int32_t enable) {
+    return guarded([&]() -> int32_t {
+        INFMOE_TRY(check(p));
+        return p->layer->setTiming(enable != 0);
+    });
+}
+
+int32_t infmoe_last_timing(infmoe_plugin* p, float* ms) {
+    return guarded([&]() -> int32_t {
+        INFMOE_TRY(check(p));
+        if (ms == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null output pointer");
+        return p->layer->lastTiming(ms);
+    });
+}
+
 int32_t infmoe_serialization_size(const infmoe_plugin* p, size_t* out_bytes) {
     return guarded([&]() -> int32_t {
         INFMOE_TRY(check(p));

@@ -229,6 +229,9 @@ Status MoELayer::terminate() {
         for (auto e : *v) (void)hipEventDestroy(e);
         v->clear();
     }
+    for (auto e : mMarks) (void)hipEventDestroy(e);
+    mMarks.clear();
+    mTimed = false;
     if (mFork) (void)hipEventDestroy(mFork);
     if (mRoutingDone) (void)hipEventDestroy(mRoutingDone);
     mFork = mRoutingDone = nullptr;
@@ -258,18 +261,27 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     int32_t* dStats = dOffset + E + 1;
     mSublayer->setLayerTokenCount(T);
 
+    const bool timed = mTiming && !mMarks.empty();
+    auto mark = [&](int i) -> Status {
+        if (timed) INFMOE_HIP(hipEventRecord(mMarks[i], stream));
+        return INFMOE_OK;
+    };
+    INFMOE_TRY(mark(0));
     // 0-2. norm (cpm_2: for scoring only), scores, top-1          plugin/MoELayerPlugin.cc:312-345
     INFMOE_HIP(launch_fill_i32(dStats, 4, 0, stream));
     const bool ln = mParams.flags.layernormOnInputBeforeScore;
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
                                 mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream));
+    INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     const bool grouped = resident();
     const int skinnyMax = grouped ? mSublayer->skinnyMaxRows(T) : 0;
     INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, grouped ? c.tiles : nullptr,
                                    grouped ? c.nTiles : nullptr, kGemmTileRows, skinnyMax, c.rowExpert, stream));
+    INFMOE_TRY(mark(2));
     INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream));  // experts see the raw input (:354)
     INFMOE_HIP(hipEventRecord(mRoutingDone, stream));
+    INFMOE_TRY(mark(3));
 
     // 4. experts                                                   plugin/MoELayerPlugin.cc:360-402
     if (grouped) {
@@ -277,10 +289,14 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
         g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
         g.tiles = c.tiles, g.nTiles = c.nTiles, g.maxTiles = c.maxTiles, g.stream = stream;
+        if (timed) g.afterNorm = mMarks[4], g.afterGemm1 = mMarks[5];
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {
+        INFMOE_TRY(mark(4));
         INFMOE_TRY(runStreamed(T, c, stream));
+        INFMOE_TRY(mark(5));
     }
+    INFMOE_TRY(mark(6));
 
     // 6-7. mix (base_layer) and un-shuffle                         plugin/MoELayerPlugin.cc:404-412
     // (the post-expert rows are gathered; :411 of the public reference passes the pre-expert ones)
@@ -288,6 +304,29 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         INFMOE_HIP(launch_mix_gather(T, d, c.pos, c.routed, c.post, c.routedCoeff, y, stream));
     else
         INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream));
+    INFMOE_TRY(mark(7));
+    mTimed = timed;
+    return INFMOE_OK;
+}
+
+Status MoELayer::setTiming(bool enable) {
+    if (enable && mMarks.empty()) {
+        mMarks.resize(INFMOE_N_PHASES + 1);
+        for (auto& e : mMarks) INFMOE_HIP(hipEventCreate(&e));
+    }
+    mTiming = enable;
+    mTimed = false;
+    return INFMOE_OK;
+}
+
+Status MoELayer::lastTiming(float* ms) {
+    if (!mTimed) return fail(INFMOE_ERR_STATE, "no timed enqueue to report (infmoe_set_timing, then infmoe_enqueue)");
+    INFMOE_HIP(hipEventSynchronize(mMarks[INFMOE_N_PHASES]));
+    for (int i = 0; i < INFMOE_N_PHASES; ++i) {
+        ms[i] = 0.f;
+        // an Identity sub-layer or a streamed expert loop leaves some marks unrecorded in this call
+        if (hipEventElapsedTime(&ms[i], mMarks[i], mMarks[i + 1]) != hipSuccess) ms[i] = 0.f;
+    }
     return INFMOE_OK;
 }
 

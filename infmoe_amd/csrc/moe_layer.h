@@ -44,6 +44,8 @@ class MoELayer {
     Status terminate();                                                        // :203-237
     Status setScoreBias(const float* host);
     Status lastRouting(int32_t* countHost, int32_t* statsHost);
+    Status setTiming(bool enable);
+    Status lastTiming(float* ms);
 
     Status serializationSize(size_t* bytes) const;
     Status serialize(void* buffer, size_t bytes) const;
@@ -76,6 +78,8 @@ class MoELayer {
     std::vector<hipStream_t> mComputeStreams;
     std::vector<hipEvent_t> mCopyDone, mComputeDone, mJoin;
     hipEvent_t mFork = nullptr, mRoutingDone = nullptr;
+    bool mTiming = false, mTimed = false;
+    std::vector<hipEvent_t> mMarks;  // INFMOE_N_PHASES + 1 phase boundaries
 };
 
 }  // namespace infmoe

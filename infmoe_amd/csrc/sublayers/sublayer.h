@@ -35,6 +35,8 @@ struct GroupedRun {
     const int32_t* nTiles = nullptr;
     int32_t maxTiles = 0;
     hipStream_t stream = nullptr;
+    // optional phase marks: recorded on `stream` after the norm and after the first GEMM
+    hipEvent_t afterNorm = nullptr, afterGemm1 = nullptr;
 };
 
 class MoESubLayer {

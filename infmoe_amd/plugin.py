@@ -71,6 +71,16 @@ class Plugin:
         capi.check(self._lib.infmoe_last_routing(self._h, count, stats))
         return np.array(count[:], np.int32), dict(near_ties=stats[0], nan_rows=stats[1], rescored=stats[2])
 
+    PHASES = ("gating", "count_sort", "scatter", "expert_norm", "expert_gemm1", "expert_gemm2", "gather")
+
+    def set_timing(self, enable: bool) -> None:
+        capi.check(self._lib.infmoe_set_timing(self._h, int(enable)))
+
+    def last_timing(self) -> dict:
+        ms = (C.c_float * len(self.PHASES))()
+        capi.check(self._lib.infmoe_last_timing(self._h, ms))
+        return dict(zip(self.PHASES, ms[:]))
+
     def clone(self) -> "Plugin":
         out = C.c_void_p()
         capi.check(self._lib.infmoe_clone(self._h, C.byref(out)))
