@@ -40,10 +40,17 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int*
     for (int e = threadIdx.x; e < E; e += kThreads) blockhist[(size_t)blockIdx.x * E + e] = s_hist[e];
 }
 
+constexpr int kMaxSortedTiles = 1024;  // row tiles the scan orders by cost; beyond that they stay in expert order
+
+// `tiles` holds 2*max_tiles entries: the schedule first, then the raw list in expert order.
+// `sched` holds kSchedInts ints: [0] number of row tiles, [1 + x] first tile of XCD x (x = 0..8).
 __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, int* __restrict__ blockhist,
                                                         int* __restrict__ count, int* __restrict__ offset,
-                                                        RowTile* __restrict__ tiles, int* __restrict__ n_tiles,
-                                                        int tile_rows, int skinny_max) {
+                                                        RowTile* __restrict__ tiles, int* __restrict__ sched,
+                                                        int max_tiles, int xcd_cap, int tile_rows, int skinny_max) {
+    __shared__ int s_n;
+    __shared__ int s_cost[kMaxSortedTiles], s_order[kMaxSortedTiles];
+    __shared__ unsigned char s_bin[kMaxSortedTiles];
     for (int e = threadIdx.x; e < E; e += kThreads) {
         int run = 0;
         for (int b = 0; b < nblk; ++b) {
@@ -54,6 +61,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, 
         count[e] = run;
     }
     __syncthreads();
+    RowTile* raw = tiles ? tiles + max_tiles : nullptr;
     if (threadIdx.x == 0) {
         int off = 0, nt = 0;
         for (int e = 0; e < E; ++e) {
@@ -66,13 +74,60 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, 
                     rt.row0 = off + m0;
                     rt.rows = min(tile_rows, c - m0);
                     rt.pad = 0;
-                    tiles[nt++] = rt;
+                    raw[nt++] = rt;
                 }
             }
             off += c;
         }
         offset[E] = off;  // == T (plugin/MoELayerPlugin.cc:351)
-        if (n_tiles != nullptr) *n_tiles = nt;
+        s_n = nt;
+    }
+    __syncthreads();
+    if (tiles == nullptr) return;
+    const int n = s_n;
+    if (n > kMaxSortedTiles) {  // many tiles balance by themselves: equal contiguous shares
+        for (int j = threadIdx.x; j < n; j += kThreads) tiles[j] = raw[j];
+        if (threadIdx.x <= kXcdCount) sched[1 + threadIdx.x] = (int)(((long long)n * threadIdx.x) / kXcdCount);
+        if (threadIdx.x == 0) sched[0] = n;
+        return;
+    }
+    // Longest-processing-time-first over the 8 XCDs: order the tiles by padded height (the cost of
+    // a tile), then give each to the least loaded XCD.  Inside an XCD the order stays descending,
+    // so the short tiles fill the tail.
+    for (int j = threadIdx.x; j < n; j += kThreads) s_cost[j] = (raw[j].rows + 15) >> 4;
+    __syncthreads();
+    for (int j = threadIdx.x; j < n; j += kThreads) {
+        const int cj = s_cost[j];
+        int rank = 0;
+        for (int i = 0; i < n; ++i) rank += (s_cost[i] > cj) || (s_cost[i] == cj && i < j);
+        s_order[rank] = j;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int load[kXcdCount], cnt[kXcdCount];
+        for (int x = 0; x < kXcdCount; ++x) load[x] = 0, cnt[x] = 0;
+        for (int r = 0; r < n; ++r) {
+            const int j = s_order[r];
+            int best = -1;
+            for (int x = 0; x < kXcdCount; ++x)
+                if (cnt[x] < xcd_cap && (best < 0 || load[x] < load[best])) best = x;
+            if (best < 0) best = r % kXcdCount;  // cannot happen while 8 * xcd_cap >= n
+            s_bin[j] = (unsigned char)best;
+            load[best] += s_cost[j];
+            cnt[best]++;
+        }
+        int start = 0;
+        sched[0] = n;
+        for (int x = 0; x < kXcdCount; ++x) {
+            sched[1 + x] = start;
+            load[x] = start;  // reused as the fill cursor
+            start += cnt[x];
+        }
+        sched[1 + kXcdCount] = start;
+        for (int r = 0; r < n; ++r) {
+            const int j = s_order[r];
+            tiles[load[s_bin[j]]++] = raw[j];
+        }
     }
 }
 
@@ -217,14 +272,15 @@ size_t expert_count_scratch_bytes(int T, int E) {
 }
 
 hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
-                               RowTile* tiles, int* n_tiles, int tile_rows, int skinny_max, int* row_expert,
+                               RowTile* tiles, int* sched, int tile_rows, int skinny_max, int* row_expert,
                                hipStream_t stream) {
     const int nblk = (T + kCountBlockTokens - 1) / kCountBlockTokens;
     int* blockhist = static_cast<int*>(scratch);
     const size_t lds = (size_t)E * sizeof(int);
     if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
-    scan_kernel<<<1, kThreads, 0, stream>>>(T, E, nblk, blockhist, count, offset, tiles, n_tiles, tile_rows,
-                                            skinny_max);
+    const int max_tiles = max_row_tiles(T, E, tile_rows);
+    scan_kernel<<<1, kThreads, 0, stream>>>(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles,
+                                            xcd_tile_capacity(max_tiles), tile_rows, skinny_max);
     if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);
     return hipGetLastError();
 }

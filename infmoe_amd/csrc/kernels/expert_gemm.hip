@@ -15,9 +15,9 @@
 // up to a whole fixed-height tile.  The 4 waves of a workgroup split the BN columns; each keeps
 // NMB x (BN/64) accumulator blocks in registers.
 //
-// Pipeline.  K advances in steps of 32 floats.  Global loads of step s+1 are issued into registers
-// before the matrix-core work of step s and written to the other half of a double-buffered LDS
-// tile afterwards; one barrier per step.  LDS rows are padded to 36 floats so that the 16-byte
+// Pipeline.  K advances in steps of 32 floats.  Global loads of step s+2 are issued into registers
+// before the matrix-core work of step s; the registers holding step s+1 are written to the other
+// half of a double-buffered LDS tile afterwards; one barrier per step.  LDS rows are padded to 36 floats so that the 16-byte
 // operand reads of the 16 lanes of a block hit distinct banks.  Inside a 16-float chunk the k order
 // is permuted identically for A and B (lane q supplies floats 4q..4q+3 over four instructions),
 // which a dot product does not see and which lets every operand read be a ds_read_b128.
@@ -29,6 +29,8 @@
 // in one XCD's L2.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernels.h"
 
 namespace infmoe {
@@ -39,7 +41,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int BK = 32;            // k floats per pipeline step
 constexpr int LDK = BK + 4;       // padded LDS row (floats)
 constexpr int kThreads = 256;     // 4 waves
-constexpr int kXcd = 8;
 
 __device__ __forceinline__ float gelu_dot(float a, float b) {
     // plugin/cuda/ops/gelu.cu:8-15
@@ -88,45 +89,41 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         if (GATED) b_ptr[NB - 1][p] = B1 + off;
     }
 
-    v4f ra[A_LOADS], rb[NB][B_LOADS];
-    auto load_global = [&](int k0) {
+    // Two register sets: global loads run two K steps ahead of the matrix core, which covers the
+    // latency of an HBM miss (every weight load is one) with two steps of MFMA work.
+    v4f ra[2][A_LOADS], rb[2][NB][B_LOADS];
+    auto load_global = [&](auto setc, int k0) {
+        constexpr int P = decltype(setc)::value;
         const bool kin = (k0 + 4 * ld_c4) < K;  // K % 4 == 0: a float4 is inside or outside as a whole
 #pragma unroll
         for (int p = 0; p < A_LOADS; ++p) {
-            ra[p] = v4f{0.f, 0.f, 0.f, 0.f};
-            if (kin && (A_ROWS % 32 == 0 || p * 32 + ld_row < A_ROWS)) ra[p] = *reinterpret_cast<const v4f*>(a_ptr[p] + k0);
+            ra[P][p] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (kin && (A_ROWS % 32 == 0 || p * 32 + ld_row < A_ROWS))
+                ra[P][p] = *reinterpret_cast<const v4f*>(a_ptr[p] + k0);
         }
 #pragma unroll
         for (int m = 0; m < NB; ++m)
 #pragma unroll
             for (int p = 0; p < B_LOADS; ++p) {
-                rb[m][p] = v4f{0.f, 0.f, 0.f, 0.f};
-                if (kin) rb[m][p] = *reinterpret_cast<const v4f*>(b_ptr[m][p] + k0);
+                rb[P][m][p] = v4f{0.f, 0.f, 0.f, 0.f};
+                if (kin) rb[P][m][p] = *reinterpret_cast<const v4f*>(b_ptr[m][p] + k0);
             }
     };
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](auto setc, int buf) {
+        constexpr int P = decltype(setc)::value;
         float* a = As + buf * a_buf;
         float* b = Bs + buf * b_buf;
 #pragma unroll
         for (int p = 0; p < A_LOADS; ++p)
             if (A_ROWS % 32 == 0 || p * 32 + ld_row < A_ROWS)
-                *reinterpret_cast<v4f*>(a + (p * 32 + ld_row) * LDK + 4 * ld_c4) = ra[p];
+                *reinterpret_cast<v4f*>(a + (p * 32 + ld_row) * LDK + 4 * ld_c4) = ra[P][p];
 #pragma unroll
         for (int m = 0; m < NB; ++m)
 #pragma unroll
             for (int p = 0; p < B_LOADS; ++p)
-                *reinterpret_cast<v4f*>(b + (m * BN + p * 32 + ld_row) * LDK + 4 * ld_c4) = rb[m][p];
+                *reinterpret_cast<v4f*>(b + (m * BN + p * 32 + ld_row) * LDK + 4 * ld_c4) = rb[P][m][p];
     };
-
-    const int nk = (K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-
-    for (int s = 0; s < nk; ++s) {
-        const int buf = s & 1;
-        if (s + 1 < nk) load_global((s + 1) * BK);
-
+    auto compute = [&](int buf) {
         const float* a = As + buf * a_buf + i * LDK + 4 * kq;
         const float* b = Bs + buf * b_buf + (wave * (BN / 4) + i) * LDK + 4 * kq;
 #pragma unroll
@@ -153,9 +150,26 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
                     }
             }
         }
-
-        if (s + 1 < nk) store_lds(buf ^ 1);
+    };
+    // Step s computes from LDS buffer s & 1 while register set P holds step s + 1 and the other
+    // set receives step s + 2; the loop is unrolled by two so that P is a compile-time constant.
+    const int nk = (K + BK - 1) / BK;
+    auto step = [&](auto setc, int s) {
+        constexpr int P = decltype(setc)::value;
+        if (s + 2 < nk) load_global(std::integral_constant<int, 1 - P>{}, (s + 2) * BK);
+        compute(s & 1);
+        if (s + 1 < nk) store_lds(setc, (s + 1) & 1);
         __syncthreads();
+    };
+    const std::integral_constant<int, 0> set0{};
+    const std::integral_constant<int, 1> set1{};
+    load_global(set1, 0);
+    store_lds(set1, 0);
+    if (nk > 1) load_global(set0, BK);
+    __syncthreads();
+    for (int s = 0; s < nk; s += 2) {
+        step(set0, s);
+        if (s + 1 < nk) step(set1, s + 1);
     }
 
     // epilogue: accumulator register r of block (mb, nb) is C[16*mb + 4*kq + r][16*nb + i]
@@ -187,9 +201,12 @@ template <int BN, bool GATED>
 __device__ __forceinline__ void gemm_dispatch(int nmb, const float* A, const float* R, float* C, int rows,
                                               const float* B0, const float* B1, int n0, int N, int K, int epilogue,
                                               float* smem, int a_alloc_rows) {
+    // the gated form keeps two accumulator sets, so its tiles are half as tall
+    constexpr int kMaxMb = (GATED ? kGemmTileRowsGated : kGemmTileRows) / 16;
 #define INFMOE_CASE(n)                                                                                       \
     case n:                                                                                                  \
-        gemm_tile<n, BN, GATED>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);              \
+        if constexpr (n <= kMaxMb)                                                                           \
+            gemm_tile<n, BN, GATED>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);          \
         break;
     switch (nmb) {
         INFMOE_CASE(1) INFMOE_CASE(2) INFMOE_CASE(3) INFMOE_CASE(4) INFMOE_CASE(5) INFMOE_CASE(6) INFMOE_CASE(7)
@@ -204,33 +221,34 @@ __device__ __forceinline__ void gemm_dispatch(int nmb, const float* A, const flo
 template <int BN, bool GATED>
 __global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, int rows_total, int a_alloc_rows) {
     extern __shared__ __align__(16) float smem[];
-    const int row0 = blockIdx.y * kGemmTileRows;
-    const int rows = min(kGemmTileRows, rows_total - row0);
+    constexpr int kTile = GATED ? kGemmTileRowsGated : kGemmTileRows;
+    const int row0 = blockIdx.y * kTile;
+    const int rows = min(kTile, rows_total - row0);
     const int n0 = blockIdx.x * BN;
     gemm_dispatch<BN, GATED>((rows + 15) >> 4, p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
                              p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K, p.epilogue, smem,
                              a_alloc_rows);
 }
 
-// All experts: 1-D grid of n_col_tiles * max_tiles workgroups.
+// All experts: 1-D grid of 8 * (row-tile capacity of an XCD) * n_col_tiles workgroups.  Workgroup id
+// b runs on XCD b % 8 and takes slot b / 8 of that XCD's share of the schedule: the share's row
+// tiles in descending height, all column tiles of a row tile in a row (they share its activations).
 template <int BN, bool GATED>
 __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProblem p, size_t weight_stride,
                                                                        const RowTile* __restrict__ tiles,
-                                                                       const int* __restrict__ n_tiles,
+                                                                       const int* __restrict__ sched,
                                                                        int n_col_tiles) {
     extern __shared__ __align__(16) float smem[];
-    const int total = *n_tiles * n_col_tiles;
-    const int per_xcd = (total + kXcd - 1) / kXcd;
-    const int xcd = blockIdx.x % kXcd, slot = blockIdx.x / kXcd;
-    const int logical = xcd * per_xcd + slot;
-    if (slot >= per_xcd || logical >= total) return;
-    const RowTile rt = tiles[logical / n_col_tiles];
-    const int n0 = (logical % n_col_tiles) * BN;
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
+    if (slot >= share * n_col_tiles) return;
+    const RowTile rt = tiles[first + slot / n_col_tiles];
+    const int n0 = (slot % n_col_tiles) * BN;
     const float* B0 = p.B + (size_t)rt.expert * weight_stride;
     const float* B1 = GATED ? p.B1 + (size_t)rt.expert * weight_stride : nullptr;
     gemm_dispatch<BN, GATED>((rt.rows + 15) >> 4, p.A + (size_t)rt.row0 * p.K,
                              p.R ? p.R + (size_t)rt.row0 * p.N : nullptr, p.C + (size_t)rt.row0 * p.N, rt.rows, B0,
-                             B1, n0, p.N, p.K, p.epilogue, smem, kGemmTileRows);
+                             B1, n0, p.N, p.K, p.epilogue, smem, GATED ? kGemmTileRowsGated : kGemmTileRows);
 }
 
 // Shapes the matrix-core kernel does not take (K not a multiple of 4, or operands that are not
@@ -283,12 +301,13 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
         expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows);
         return hipGetLastError();
     }
-    const int a_alloc = min(kGemmTileRows, ((rows + 15) / 16) * 16);
-    const dim3 grid((p.N + kBN - 1) / kBN, (rows + kGemmTileRows - 1) / kGemmTileRows);
+    const int tile = gemm_tile_rows(p.epilogue);
+    const int a_alloc = min(tile, ((rows + 15) / 16) * 16);
+    const dim3 grid((p.N + kBN - 1) / kBN, (rows + tile - 1) / tile);
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
         const size_t lds = lds_bytes<kBN, true>(a_alloc);
-        if ((err = allow_lds(expert_gemm_kernel<kBN, true>, lds_bytes<kBN, true>(kGemmTileRows))) != hipSuccess) return err;
+        if ((err = allow_lds(expert_gemm_kernel<kBN, true>, lds_bytes<kBN, true>(kGemmTileRowsGated))) != hipSuccess) return err;
         expert_gemm_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, rows, a_alloc);
     } else {
         const size_t lds = lds_bytes<kBN, false>(a_alloc);
@@ -299,21 +318,20 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
 }
 
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
-                                      const int* n_tiles, int max_tiles, hipStream_t stream) {
+                                      const int* sched, int max_tiles, hipStream_t stream) {
     if (max_tiles <= 0) return hipSuccess;
     if (!fast_path_ok(p) || weight_stride % 4 != 0) return hipErrorInvalidValue;  // callers fall back per expert
     const int n_col_tiles = (p.N + kBN - 1) / kBN;
-    const int total = n_col_tiles * max_tiles;
-    const dim3 grid(((total + kXcd - 1) / kXcd) * kXcd);
+    const dim3 grid((unsigned)kXcdCount * (unsigned)xcd_tile_capacity(max_tiles) * (unsigned)n_col_tiles);
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
-        const size_t lds = lds_bytes<kBN, true>(kGemmTileRows);
+        const size_t lds = lds_bytes<kBN, true>(kGemmTileRowsGated);
         if ((err = allow_lds(expert_gemm_grouped_kernel<kBN, true>, lds)) != hipSuccess) return err;
-        expert_gemm_grouped_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, n_tiles, n_col_tiles);
+        expert_gemm_grouped_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     } else {
         const size_t lds = lds_bytes<kBN, false>(kGemmTileRows);
         if ((err = allow_lds(expert_gemm_grouped_kernel<kBN, false>, lds)) != hipSuccess) return err;
-        expert_gemm_grouped_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, n_tiles, n_col_tiles);
+        expert_gemm_grouped_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     }
     return hipGetLastError();
 }

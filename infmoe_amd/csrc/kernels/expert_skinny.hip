@@ -4,15 +4,21 @@
 // calls of plugin/sublayers/T5FFLayer.cc:112-138), but with so few activation rows the work is a
 // stream of the expert's weights through the chip: 2*d*h*4 bytes per expert, each byte used once
 // per row.  The kernel is therefore built around bytes in flight, not around the matrix core:
-//   * a workgroup owns 32 weight rows (8 per wave) and walks K in chunks of 2048 floats;
-//   * the activation chunk (M x 2048 floats) is staged in LDS once per chunk and shared by all
-//     32 weight rows, so activations cost L2/LDS bandwidth only;
-//   * every lane keeps 16 independent 16-byte weight loads in flight (two weight rows x eight
-//     1-KB wave-wide segments), and several workgroups are resident per CU;
+//   * a wave owns 8 weight rows and walks K in chunks; no LDS and no barrier, so waves never wait
+//     for each other and occupancy is bounded by registers only;
+//   * the activation chunk (M rows) lives in registers, loaded once per chunk from L2 and reused
+//     for the wave's 8 weight rows;
+//   * every lane keeps 8-16 independent 16-byte weight loads in flight (whole 1-KB wave-wide
+//     segments of 2-8 weight rows), marked non-temporal: each weight byte is used once, and the
+//     register budget is capped so that three waves share a SIMD (12 waves x 16 KB per CU);
 //   * partial dot products stay in registers across chunks and are reduced across the wave once.
+// The chunk length shrinks as M grows (2048, 2048, 512, 256 floats for M = 1, 2, 4, 8) so that
+// activations + loads in flight + accumulators stay within 168 registers.
 // Experts outside 1..kSkinnyMaxRows rows are skipped, so the grouped launch can run next to the
 // matrix-core launch: each expert is processed by exactly one of the two.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -22,11 +28,8 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int KC = 2048;            // K floats per staged chunk
-constexpr int KC4 = KC / 4;
 constexpr int RW = 8;               // weight rows per wave
 constexpr int kRowsPerWg = RW * (kThreads / 64);
-constexpr int kSeg = KC / 256;      // 16-byte loads per lane per weight row per chunk
 
 __device__ __forceinline__ float gelu_dot(float a, float b) {
     // plugin/cuda/ops/gelu.cu:8-15
@@ -40,15 +43,20 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-template <int M, bool GATED>
+// SEG: 16-byte loads per lane per weight row per chunk; RPN: weight rows loaded together
+template <int M, int SEG, int RPN, bool GATED>
 __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const float* __restrict__ R,
                                             float* __restrict__ C, int rows, const float* __restrict__ B0,
-                                            const float* __restrict__ B1, int N, int K, int epilogue,
-                                            float* __restrict__ smem) {
+                                            const float* __restrict__ B1, int N, int K, int epilogue) {
     constexpr int NB = GATED ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int KC = SEG * 256;                   // k floats per chunk
+    constexpr int RP = RPN / NB > 0 ? RPN / NB : 1;
+    static_assert(RW % RP == 0, "bad chunking");
+    // the wave index is uniform: as a scalar it lets every row base live in SGPRs, so a load needs
+    // only the lane's 32-bit offset instead of a 64-bit address per (row, segment)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_base = blockIdx.x * kRowsPerWg + wave * RW;
-    v4f* As4 = reinterpret_cast<v4f*>(smem);  // [M][KC4]
+    if (n_base >= N) return;  // no barriers in this kernel: a wave may leave early
 
     float acc[NB][RW][M];
 #pragma unroll
@@ -58,47 +66,62 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
 #pragma unroll
             for (int m = 0; m < M; ++m) acc[b][r][m] = 0.f;
 
-    for (int kc0 = 0; kc0 < K; kc0 += KC) {
-        __syncthreads();  // everyone is done with the previous chunk
-        for (int idx = tid; idx < M * KC4; idx += kThreads) {
-            const int m = idx / KC4, c = idx - m * KC4;
-            const int k = kc0 + 4 * c;
-            v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (k < K) v = *reinterpret_cast<const v4f*>(A + (size_t)min(m, rows - 1) * K + k);
-            As4[idx] = v;
+    // Whole chunks of K: every load is unconditional and issued back to back.
+    auto chunk = [&](int kc0) {
+        v4f a[M][SEG];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const v4f* pa = reinterpret_cast<const v4f*>(A + (size_t)min(m, rows - 1) * K + kc0) + lane;
+#pragma unroll
+            for (int j = 0; j < SEG; ++j) a[m][j] = pa[64 * j];
         }
-        __syncthreads();
-
 #pragma unroll
-        for (int rp = 0; rp < RW; rp += 2) {
-            v4f w[NB][2][kSeg];
+        for (int rp = 0; rp < RW; rp += RP) {
+            v4f w[NB][RP][SEG];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const size_t roff = (size_t)min(n_base + rp + q, N - 1) * K;
+            for (int q = 0; q < RP; ++q) {
+                const size_t roff = (size_t)min(n_base + rp + q, N - 1) * K + kc0;
+                const v4f* pb0 = reinterpret_cast<const v4f*>(B0 + roff) + lane;
+                const v4f* pb1 = GATED ? reinterpret_cast<const v4f*>(B1 + roff) + lane : nullptr;
 #pragma unroll
-                for (int j = 0; j < kSeg; ++j) {
-                    const int k = kc0 + 4 * (lane + 64 * j);
-                    w[0][q][j] = v4f{0.f, 0.f, 0.f, 0.f};
-                    if (GATED) w[NB - 1][q][j] = v4f{0.f, 0.f, 0.f, 0.f};
-                    if (k < K) {
-                        w[0][q][j] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(B0 + roff + k));
-                        if (GATED) w[NB - 1][q][j] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(B1 + roff + k));
-                    }
+                for (int j = 0; j < SEG; ++j) {
+                    w[0][q][j] = __builtin_nontemporal_load(pb0 + 64 * j);
+                    if (GATED) w[NB - 1][q][j] = __builtin_nontemporal_load(pb1 + 64 * j);
                 }
             }
 #pragma unroll
-            for (int j = 0; j < kSeg; ++j) {
+            for (int q = 0; q < RP; ++q)
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    const v4f a = As4[m * KC4 + lane + 64 * j];
+                for (int j = 0; j < SEG; ++j)
 #pragma unroll
-                    for (int b = 0; b < NB; ++b)
+                    for (int b = 0; b < NB; ++b) {
+                        const v4f x = w[b][q][j];
 #pragma unroll
-                        for (int q = 0; q < 2; ++q) {
-                            const v4f x = w[b][q][j];
-                            acc[b][rp + q][m] += (x.x * a.x + x.y * a.y) + (x.z * a.z + x.w * a.w);
-                        }
-                }
+                        for (int m = 0; m < M; ++m)
+                            acc[b][rp + q][m] += (x.x * a[m][j].x + x.y * a[m][j].y) + (x.z * a[m][j].z + x.w * a[m][j].w);
+                    }
+            // keep the next group's loads behind this group's arithmetic: hoisting them all to the
+            // top of the chunk would need four times the registers and cost occupancy
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int kc0 = 0;
+    for (; kc0 + KC <= K; kc0 += KC) chunk(kc0);
+    // what is left of an odd K (K % 4 == 0): one float4 per lane and step, kept deliberately small
+#pragma unroll 1
+    for (int k = kc0 + 4 * lane; k < K; k += 256) {
+        v4f a[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) a[m] = *reinterpret_cast<const v4f*>(A + (size_t)min(m, rows - 1) * K + k);
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            const size_t roff = (size_t)min(n_base + r, N - 1) * K + k;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const v4f x = *reinterpret_cast<const v4f*>((b == 0 ? B0 : B1) + roff);
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                    acc[b][r][m] += (x.x * a[m].x + x.y * a[m].y) + (x.z * a[m].z + x.w * a[m].w);
             }
         }
     }
@@ -127,10 +150,9 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
 
 // count == nullptr: one expert with `rows_fixed` rows at row 0; else blockIdx.y is the expert.
 template <bool GATED>
-__global__ __launch_bounds__(kThreads) void expert_skinny_kernel(GemmProblem p, size_t weight_stride,
+__global__ __launch_bounds__(kThreads, 3) void expert_skinny_kernel(GemmProblem p, size_t weight_stride,
                                                                  const int* __restrict__ count,
                                                                  const int* __restrict__ offset, int rows_fixed) {
-    extern __shared__ __align__(16) float smem[];
     int rows = rows_fixed, row0 = 0;
     const float* B0 = p.B;
     const float* B1 = p.B1;
@@ -146,18 +168,13 @@ __global__ __launch_bounds__(kThreads) void expert_skinny_kernel(GemmProblem p, 
     const float* R = p.R ? p.R + (size_t)row0 * p.N : nullptr;
     float* C = p.C + (size_t)row0 * p.N;
     if (rows == 1)
-        skinny_body<1, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue, smem);
+        skinny_body<1, 8, 2, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue);
     else if (rows == 2)
-        skinny_body<2, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue, smem);
+        skinny_body<2, 8, 2, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue);
     else if (rows <= 4)
-        skinny_body<4, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue, smem);
+        skinny_body<4, 2, 8, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue);
     else
-        skinny_body<8, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue, smem);
-}
-
-inline size_t lds_for_rows(int rows) {
-    const int m = rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8;
-    return (size_t)m * KC * sizeof(float);
+        skinny_body<8, 1, 8, GATED>(A, R, C, rows, B0, B1, p.N, p.K, p.epilogue);
 }
 
 bool fast_path_ok(const GemmProblem& p) {
@@ -172,11 +189,10 @@ hipError_t launch_expert_skinny(const GemmProblem& p, int rows, hipStream_t stre
     if (rows <= 0) return hipSuccess;
     if (rows > kSkinnyMaxRows || !fast_path_ok(p)) return hipErrorInvalidValue;
     const dim3 grid((p.N + kRowsPerWg - 1) / kRowsPerWg, 1);
-    const size_t lds = lds_for_rows(rows);
     if (p.epilogue == EPI_GATED_GELU)
-        expert_skinny_kernel<true><<<grid, kThreads, lds, stream>>>(p, 0, nullptr, nullptr, rows);
+        expert_skinny_kernel<true><<<grid, kThreads, 0, stream>>>(p, 0, nullptr, nullptr, rows);
     else
-        expert_skinny_kernel<false><<<grid, kThreads, lds, stream>>>(p, 0, nullptr, nullptr, rows);
+        expert_skinny_kernel<false><<<grid, kThreads, 0, stream>>>(p, 0, nullptr, nullptr, rows);
     return hipGetLastError();
 }
 
@@ -185,11 +201,10 @@ hipError_t launch_expert_skinny_grouped(const GemmProblem& p, size_t weight_stri
     if (E <= 0) return hipSuccess;
     if (!fast_path_ok(p) || weight_stride % 4 != 0) return hipErrorInvalidValue;
     const dim3 grid((p.N + kRowsPerWg - 1) / kRowsPerWg, E);
-    const size_t lds = lds_for_rows(kSkinnyMaxRows);
     if (p.epilogue == EPI_GATED_GELU)
-        expert_skinny_kernel<true><<<grid, kThreads, lds, stream>>>(p, weight_stride, count, offset, 0);
+        expert_skinny_kernel<true><<<grid, kThreads, 0, stream>>>(p, weight_stride, count, offset, 0);
     else
-        expert_skinny_kernel<false><<<grid, kThreads, lds, stream>>>(p, weight_stride, count, offset, 0);
+        expert_skinny_kernel<false><<<grid, kThreads, 0, stream>>>(p, weight_stride, count, offset, 0);
     return hipGetLastError();
 }
 

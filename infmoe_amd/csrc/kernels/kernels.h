@@ -31,13 +31,22 @@ struct RowTile {
 };
 constexpr int kCountBlockTokens = 1024;  // tokens ranked by one workgroup
 size_t expert_count_scratch_bytes(int T, int E);
+constexpr int kXcdCount = 8;    // accelerator dies of an MI355X; workgroup ids are dealt to them round-robin
+constexpr int kSchedInts = 16;  // [0] number of row tiles, [1..9] first tile of each XCD's share
+inline int max_row_tiles(int T, int E, int tile_rows) { return (T + tile_rows - 1) / tile_rows + E; }
+// Most row tiles one XCD may be given (bounds the grid of the grouped launch).
+inline int xcd_tile_capacity(int max_tiles) {
+    const int cap = 2 * ((max_tiles + kXcdCount - 1) / kXcdCount) + 8;
+    return cap < max_tiles ? cap : max_tiles;
+}
 // Optional outputs for the grouped expert launch (all may be null):
-//   tiles/n_tiles: row tiles of height <= tile_rows over experts with more than `skinny_max` rows
+//   tiles (2*max_row_tiles entries) / sched (kSchedInts ints): row tiles of height <= tile_rows
+//     over the experts with more than `skinny_max` rows, dealt to the 8 XCDs so that the padded
+//     row counts balance, each XCD's share in descending height
 //   row_expert[T]: expert of every routed row
 hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
-                               RowTile* tiles, int* n_tiles, int tile_rows, int skinny_max, int* row_expert,
+                               RowTile* tiles, int* sched, int tile_rows, int skinny_max, int* row_expert,
                                hipStream_t stream);
-inline int max_row_tiles(int T, int E, int tile_rows) { return (T + tile_rows - 1) / tile_rows + E; }
 
 // Small fill kernel (used instead of hipMemsetAsync so that callers may capture the layer in a graph).
 hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream);
@@ -75,8 +84,10 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
 // All experts in one launch: A, R, C address routed rows globally; expert e's weights are at
 // B + e*weight_stride (floats).  Row tiles and their number come from launch_expert_count.
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
-                                      const int* n_tiles, int max_tiles, hipStream_t stream);
-constexpr int kGemmTileRows = 256;  // tallest row tile of the GEMM kernel
+                                      const int* sched, int max_tiles, hipStream_t stream);
+constexpr int kGemmTileRows = 256;       // tallest row tile of the GEMM kernel
+constexpr int kGemmTileRowsGated = 128;  // ... of its two-matrix (gated) form
+inline int gemm_tile_rows(int epilogue) { return epilogue == EPI_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
 
 // Few-row experts (decode): every weight row is streamed once and dotted with up to
 // kSkinnyMaxRows activation rows held in LDS.

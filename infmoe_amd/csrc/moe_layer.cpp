@@ -121,7 +121,7 @@ struct MoELayer::Carve {
     char* slots = nullptr;
     size_t slotStride = 0;
     char* subWs = nullptr;
-    int32_t *sel = nullptr, *pos = nullptr, *rowExpert = nullptr, *nTiles = nullptr;
+    int32_t *sel = nullptr, *pos = nullptr, *rowExpert = nullptr, *sched = nullptr;
     RowTile* tiles = nullptr;
     int maxTiles = 0;
     void* countScratch = nullptr;
@@ -150,9 +150,9 @@ Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     c->sel = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
     c->pos = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
     c->rowExpert = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
-    c->maxTiles = max_row_tiles(T, E, kGemmTileRows);
-    c->tiles = reinterpret_cast<RowTile*>(take(sizeof(RowTile) * (size_t)c->maxTiles));
-    c->nTiles = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
+    c->maxTiles = max_row_tiles(T, E, mSublayer->rowTileHeight());
+    c->tiles = reinterpret_cast<RowTile*>(take(sizeof(RowTile) * 2 * (size_t)c->maxTiles));
+    c->sched = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kSchedInts));
     c->countScratch = take(expert_count_scratch_bytes(T, E));
     c->coeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
     c->routedCoeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
@@ -277,7 +277,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     const bool grouped = resident();
     const int skinnyMax = grouped ? mSublayer->skinnyMaxRows(T) : 0;
     INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, grouped ? c.tiles : nullptr,
-                                   grouped ? c.nTiles : nullptr, kGemmTileRows, skinnyMax, c.rowExpert, stream));
+                                   grouped ? c.sched : nullptr, mSublayer->rowTileHeight(), skinnyMax, c.rowExpert, stream));
     INFMOE_TRY(mark(2));
     INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream));  // experts see the raw input (:354)
     INFMOE_HIP(hipEventRecord(mRoutingDone, stream));
@@ -288,7 +288,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         GroupedRun g;
         g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
         g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
-        g.tiles = c.tiles, g.nTiles = c.nTiles, g.maxTiles = c.maxTiles, g.stream = stream;
+        g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
         if (timed) g.afterNorm = mMarks[4], g.afterGemm1 = mMarks[5];
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {

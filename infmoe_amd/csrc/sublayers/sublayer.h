@@ -31,9 +31,9 @@ struct GroupedRun {
     const int32_t* count = nullptr;      // [E]
     const int32_t* offset = nullptr;     // [E+1]
     const int32_t* rowExpert = nullptr;  // [T]
-    const RowTile* tiles = nullptr;      // row tiles of the experts with more than skinnyMax rows
-    const int32_t* nTiles = nullptr;
-    int32_t maxTiles = 0;
+    const RowTile* tiles = nullptr;      // scheduled row tiles of the experts with more than skinnyMax rows
+    const int32_t* sched = nullptr;      // kSchedInts ints describing the schedule
+    int32_t maxTiles = 0;                // max_row_tiles(T, E, rowTileHeight())
     hipStream_t stream = nullptr;
     // optional phase marks: recorded on `stream` after the norm and after the first GEMM
     hipEvent_t afterNorm = nullptr, afterGemm1 = nullptr;
@@ -83,6 +83,8 @@ class MoESubLayer {
     virtual size_t residentStride() const { return 0; }
     // Row-count threshold below which runGrouped handles an expert outside the row tiles.
     virtual int skinnyMaxRows(int32_t /*tokenCount*/) const { return 0; }
+    // Tallest row tile runGrouped wants the dispatch scan to cut an expert's rows into.
+    virtual int rowTileHeight() const { return kGemmTileRows; }
     virtual Status runGrouped(const GroupedRun& g) = 0;
     void setLayerTokenCount(int32_t tokens) { mLayerTokenCount = tokens; }
     int expertCount() const { return mExpertCount; }

@@ -199,10 +199,10 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     g2.epilogue = EPI_RESIDUAL;
     const bool skinny = skinnyMaxRows(T) > 0;
     if (g.afterNorm) INFMOE_HIP(hipEventRecord(g.afterNorm, g.stream));
-    INFMOE_HIP(launch_expert_gemm_grouped(g1, stride, g.tiles, g.nTiles, g.maxTiles, g.stream));
+    INFMOE_HIP(launch_expert_gemm_grouped(g1, stride, g.tiles, g.sched, g.maxTiles, g.stream));
     if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g1, stride, g.count, g.offset, mExpertCount, g.stream));
     if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, g.stream));
-    INFMOE_HIP(launch_expert_gemm_grouped(g2, stride, g.tiles, g.nTiles, g.maxTiles, g.stream));
+    INFMOE_HIP(launch_expert_gemm_grouped(g2, stride, g.tiles, g.sched, g.maxTiles, g.stream));
     if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g2, stride, g.count, g.offset, mExpertCount, g.stream));
     return INFMOE_OK;
 }

@@ -40,6 +40,7 @@ class T5FFLayer : public MoESubLayer {
     const void* residentWeights() const override { return mDeviceWeights; }
     size_t residentStride() const override { return slotStride(); }
     int skinnyMaxRows(int32_t tokenCount) const override;
+    int rowTileHeight() const override { return mFfnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
     Status runGrouped(const GroupedRun& g) override;
 
     // used by the kernel-level C entry points
