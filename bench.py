@@ -36,7 +36,7 @@ CONFIGS = {
 }
 
 
-def build_layer(torch, cfg, seed=0, keep_host=True):
+def build_layer(torch, cfg, seed=0, keep_host=True, replicate=False):
     """Synthetic tensors drawn on the GPU (fixed seed), expert weights handed to the library by
     host pointer, as a caller holding an npz in memory would."""
     from infmoe_amd import MoELayerConfig, MoELayerPlugin
@@ -56,6 +56,14 @@ def build_layer(torch, cfg, seed=0, keep_host=True):
     slots = []
     slot_floats = d + 2 * d * h
     for e in range(E):
+        if replicate and e > 0:  # profiling runs: every expert gets expert 0's values (same work, short set-up)
+            base = slots[0].ctypes.data if keep_host else slot.ctypes.data
+            plugin.set_expert_weights_ptr(e, "layer_norm_weight", base, d)
+            plugin.set_expert_weights_ptr(e, "wi_weight", base + 4 * d, d * h)
+            plugin.set_expert_weights_ptr(e, "wo_weight", base + 4 * (d + d * h), d * h)
+            if keep_host:
+                slots.append(slots[0])
+            continue
         slot = np.empty(slot_floats, np.float32)  # [gamma | wi [h][d] | wo [d][h]]
         slot[:d] = (1 + 0.1 * torch.randn(d, generator=gen, device="cuda")).cpu().numpy()
         slot[d:d + d * h] = (torch.randn(h, d, generator=gen, device="cuda") / d ** 0.5).cpu().numpy().ravel()
@@ -99,7 +107,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=int, default=1024)
+    ap.add_argument("--cpu-sample", type=int, default=4096)
+    ap.add_argument("--replicate-weights", action="store_true",
+                    help="profiling aid: give every expert the values of expert 0 (short set-up, same work)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this layer runs on one GPU; --gpus above 1 is not supported "
@@ -116,7 +126,8 @@ def main():
     B, S = cfg["shape"]
     T = B * S
     torch.cuda.set_device(0)
-    plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=not args.no_cpu)
+    plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=not args.no_cpu,
+                                                      replicate=args.replicate_weights)
     dims = [B, S, d]
     ws = torch.empty(plugin.workspace_size(dims), dtype=torch.uint8, device="cuda")
     y = torch.empty_like(x)
@@ -185,7 +196,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic",
+        "data": "synthetic" + (" (expert 0 replicated)" if args.replicate_weights else ""),
         "config": {"workload": f"{args.config}: {cfg['variant']} E={E} d={d} h={h} tokens={T} ({B}x{S}) "
                                f"max_concurrency={cfg['mc']} ({'resident' if resident else 'streamed'} experts), "
                                f"T5_FF rms norm + relu", "tokens": T, "active_experts": active,
