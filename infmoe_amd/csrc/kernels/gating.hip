@@ -4,14 +4,14 @@
 // plugin/cuda/ops/layernorm.cu:136-188, plugin/cuda/moe.cu:13-76) and removes the
 // normalised-input and score-matrix round trips through memory.
 //
-// Work split: one workgroup (4 waves) owns 16 tokens; the 4 waves split the embedding
+// Work split: one workgroup (8 waves) owns 16 tokens; the 8 waves split the embedding
 // dimension in interleaved 16-float chunks and each runs v_mfma_f32_16x16x4_f32 with the
 // tokens as the A rows and up to 128 experts (8 column blocks) as the B columns.  The row
 // statistics of the norm are accumulated from the same registers that feed the matrix core,
 // and the norm is applied to the 16xE score tile instead of to the 16xd input:
 //     rms:      score = rstd * sum_k x_k g_k c_ek
 //     centered: score = rstd * (sum_k x_k g_k c_ek - mu * sum_k g_k c_ek)
-// Partial tiles of the 4 waves meet in LDS, then each wave reduces 4 tokens to
+// Partial tiles of the 8 waves meet in LDS, then each wave reduces 2 tokens to
 // (best, index, runner-up) with the reference's tie rule (lowest index wins,
 // plugin/cuda/moe.cu:62-68).
 //
@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cfloat>
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -32,14 +33,17 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kTokens = 16;   // tokens per workgroup (MFMA M)
-constexpr int kWaves = 4;     // waves per workgroup, each takes every 4th 16-float chunk
+constexpr int kWaves = 8;     // waves per workgroup, each takes every 8th 16-float chunk
 constexpr int kThreads = 64 * kWaves;
 
+// Four floats of a row starting at k.  With VEC (d % 4 == 0, 16-byte aligned rows) the load is
+// unconditional: a k beyond the row is clamped to the last float4 and the caller discards the value
+// when it uses it, so that no load sits inside a branch and many can be in flight.
 template <bool VEC>
 __device__ __forceinline__ v4f load4(const float* __restrict__ row, int k, int d) {
     v4f v = {0.f, 0.f, 0.f, 0.f};
     if (VEC) {
-        if (k < d) v = *reinterpret_cast<const v4f*>(row + k);
+        v = *reinterpret_cast<const v4f*>(row + min(k, d - 4));
     } else {
         if (k + 0 < d) v.x = row[k + 0];
         if (k + 1 < d) v.y = row[k + 1];
@@ -56,7 +60,7 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 // NBLK: 16-expert column blocks handled per pass (experts per pass = 16*NBLK).
-template <int NBLK, bool VEC>
+template <int NBLK, bool VEC, bool GAMMA>
 __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E, const float* __restrict__ X,
                                                              const float* __restrict__ C,
                                                              const float* __restrict__ gamma, int norm_kind,
@@ -71,7 +75,8 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
     __shared__ float s_G[EP], s_cn[EP];
     __shared__ float s_best[kTokens], s_second[kTokens], s_cnmax;
     __shared__ int s_besti[kTokens], s_rescue[kTokens];
-    __shared__ double s_red[kWaves][8];
+    __shared__ double s_red[kWaves][2];
+    __shared__ double s_sc64[EP];
     __shared__ double s_bcast[2];
 
     const int tid = threadIdx.x;
@@ -81,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
     const int kq = lane >> 4;  // which float4 of the 16-float chunk this lane feeds
     const int t0 = blockIdx.x * kTokens;
     const int nchunks = (d + 15) >> 4;
-    const bool use_gamma = (norm_kind != NORM_NONE) && gamma != nullptr;
+    constexpr bool use_gamma = GAMMA;  // the norm's gamma is folded into the centroids as they are loaded
 
     if (tid < kTokens) {
         s_best[tid] = -FLT_MAX;  // plugin/cuda/moe.cu:26-27
@@ -106,25 +111,56 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
         }
         float s1 = 0.f, s2 = 0.f;
 
-        for (int c = wave; c < nchunks; c += kWaves) {
-            const int k = c * 16 + 4 * kq;
-            const v4f xv = load4<VEC>(xrow, k, d);
-            v4f gv = {1.f, 1.f, 1.f, 1.f};
-            if (use_gamma) gv = load4<VEC>(gamma, k, d);
-            s1 += (xv.x + xv.y) + (xv.z + xv.w);
-            s2 += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
+        // The wave's chunks are taken U at a time, and the loads of the next batch are issued
+        // before the arithmetic of the current one (two register sets, loop unrolled by two):
+        // without that every chunk would wait out a full memory latency.
+        constexpr int U = NBLK <= 2 ? 4 : (NBLK == 4 ? 2 : 1);
+        v4f xr[2][U], gr[2][U], cr[2][U][NBLK];
+        auto load_batch = [&](auto setc, int c0) {
+            constexpr int P = decltype(setc)::value;
 #pragma unroll
-            for (int nb = 0; nb < NBLK; ++nb) {
-                v4f cv = load4<VEC>(crow[nb], k, d);
-                cv *= gv;
-                gs[nb] += (cv.x + cv.y) + (cv.z + cv.w);
-                cn[nb] += (cv.x * cv.x + cv.y * cv.y) + (cv.z * cv.z + cv.w * cv.w);
-                // The k order inside a chunk is permuted identically for A and B, which a dot
-                // product does not see: step j multiplies element j of every lane's float4.
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.x, cv.x, acc[nb], 0, 0, 0);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.y, cv.y, acc[nb], 0, 0, 0);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.z, cv.z, acc[nb], 0, 0, 0);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.w, cv.w, acc[nb], 0, 0, 0);
+            for (int u = 0; u < U; ++u) {
+                const int k = (c0 + u * kWaves) * 16 + 4 * kq;
+                xr[P][u] = load4<VEC>(xrow, k, d);
+                gr[P][u] = v4f{1.f, 1.f, 1.f, 1.f};
+                if (use_gamma) gr[P][u] = load4<VEC>(gamma, k, d);
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) cr[P][u][nb] = load4<VEC>(crow[nb], k, d);
+            }
+        };
+        auto compute_batch = [&](auto setc, int c0) {
+            constexpr int P = decltype(setc)::value;
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool inside = (c0 + u * kWaves) * 16 + 4 * kq < d;  // beyond the row: contributes nothing
+                const v4f xv = inside ? xr[P][u] : zero, gv = gr[P][u];
+                s1 += (xv.x + xv.y) + (xv.z + xv.w);
+                s2 += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    const v4f cv = inside ? cr[P][u][nb] * gv : zero;
+                    gs[nb] += (cv.x + cv.y) + (cv.z + cv.w);
+                    cn[nb] += (cv.x * cv.x + cv.y * cv.y) + (cv.z * cv.z + cv.w * cv.w);
+                    // The k order inside a chunk is permuted identically for A and B, which a dot
+                    // product does not see: step j multiplies element j of every lane's float4.
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.x, cv.x, acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.y, cv.y, acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.z, cv.z, acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.w, cv.w, acc[nb], 0, 0, 0);
+                }
+            }
+        };
+        const std::integral_constant<int, 0> set0{};
+        const std::integral_constant<int, 1> set1{};
+        constexpr int kStride = U * kWaves;  // chunks between two batches of one wave
+        load_batch(set0, wave);
+        for (int c = wave; c < nchunks; c += 2 * kStride) {
+            if (c + kStride < nchunks) load_batch(set1, c + kStride);
+            compute_batch(set0, c);
+            if (c + kStride < nchunks) {
+                if (c + 2 * kStride < nchunks) load_batch(set0, c + 2 * kStride);
+                compute_batch(set1, c + kStride);
             }
         }
 
@@ -155,8 +191,9 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
         __syncthreads();
 
         if (tid < kTokens) {
-            const float a1 = (s_s1[0][tid] + s_s1[1][tid]) + (s_s1[2][tid] + s_s1[3][tid]);
-            const float a2 = (s_s2[0][tid] + s_s2[1][tid]) + (s_s2[2][tid] + s_s2[3][tid]);
+            float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) a1 += s_s1[w][tid], a2 += s_s2[w][tid];
             float mu = 0.f, rstd = 1.f;
             if (norm_kind == NORM_RMS) {
                 rstd = 1.0f / sqrtf(a2 / (float)d + kNormEps);
@@ -169,29 +206,34 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
             s_xnorm[tid] = sqrtf(a2);
         } else if (tid >= 64 && tid < 64 + EP) {
             const int e = tid - 64;
-            s_G[e] = (s_g1[0][e] + s_g1[1][e]) + (s_g1[2][e] + s_g1[3][e]);
-            s_cn[e] = sqrtf((s_g2[0][e] + s_g2[1][e]) + (s_g2[2][e] + s_g2[3][e]));
+            float g1 = 0.f, g2 = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) g1 += s_g1[w][e], g2 += s_g2[w][e];
+            s_G[e] = g1;
+            s_cn[e] = sqrtf(g2);
         }
         __syncthreads();
 
         for (int idx = tid; idx < kTokens * EP; idx += kThreads) {
             const int tok = idx / EP, e = idx - tok * EP;
-            float dot = (s_part[0][tok][e] + s_part[1][tok][e]) + (s_part[2][tok][e] + s_part[3][tok][e]);
+            float dot = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) dot += s_part[w][tok][e];
             float sc = s_rstd[tok] * (dot - s_mu[tok] * s_G[e]);
             if (bias != nullptr && e0 + e < E) sc += bias[e0 + e];
             s_score[tok][e] = sc;
         }
         __syncthreads();
 
-        // each wave reduces 4 tokens
+        // each wave reduces kTokens / kWaves tokens
         const int nvalid = min(E - e0, EP);
         float cmax = 0.f;
         for (int e = lane; e < nvalid; e += 64) cmax = fmaxf(cmax, s_cn[e]);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) cmax = fmaxf(cmax, __shfl_xor(cmax, off));
         if (tid == 0) s_cnmax = fmaxf(s_cnmax, cmax);
-        for (int q = 0; q < 4; ++q) {
-            const int tok = 4 * wave + q;
+        for (int q = 0; q < kTokens / kWaves; ++q) {
+            const int tok = (kTokens / kWaves) * wave + q;
             float v = -FLT_MAX;
             int vi = -1;
             for (int e = lane; e < nvalid; e += 64) {
@@ -244,14 +286,15 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
             } else {
                 sel[t] = I;
                 coeff[t] = B;
-                const float bound = 16.f * FLT_EPSILON * s_rstd[tid] * s_xnorm[tid] * s_cnmax;
+                const float bound = 8.f * FLT_EPSILON * s_rstd[tid] * s_xnorm[tid] * s_cnmax;
                 if (E > 1 && (B - S) < fmaxf(bound, 4e-6f * fabsf(B))) s_rescue[tid] = 1;
             }
         }
     }
     __syncthreads();
 
-    // ---- float64 re-scoring of the flagged tokens by the whole workgroup
+    // ---- float64 re-scoring of the flagged tokens by the whole workgroup: the waves share the
+    // row statistics, then each wave takes every kWaves-th expert and the scores meet in LDS
     for (int tok = 0; tok < kTokens; ++tok) {
         if (!s_rescue[tok]) continue;  // uniform: read from LDS after the barrier
         const int t = t0 + tok;
@@ -270,8 +313,8 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
         }
         __syncthreads();
         if (tid == 0) {
-            const double t1 = (s_red[0][0] + s_red[1][0]) + (s_red[2][0] + s_red[3][0]);
-            const double t2 = (s_red[0][1] + s_red[1][1]) + (s_red[2][1] + s_red[3][1]);
+            double t1 = 0.0, t2 = 0.0;
+            for (int w = 0; w < kWaves; ++w) t1 += s_red[w][0], t2 += s_red[w][1];
             double mu = 0.0, rstd = 1.0;
             if (norm_kind == NORM_RMS) {
                 rstd = 1.0 / sqrt(t2 / d + 1e-6);
@@ -286,27 +329,53 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
         const double mu = s_bcast[0], rstd = s_bcast[1];
         double best = -DBL_MAX, second = -DBL_MAX;
         int besti = -1;
-        for (int e0 = 0; e0 < E; e0 += 8) {
-            double a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            for (int k = tid; k < d; k += kThreads) {
-                const double xv = ((double)xr[k] - mu) * (use_gamma ? (double)gamma[k] : 1.0);
+        for (int e0 = 0; e0 < E; e0 += EP) {
+            const int nvalid = min(E - e0, EP);
+            // wave w scores experts w, w + kWaves, ... of this pass; the k loop is outside so that
+            // x and gamma are loaded once per slice and all of the wave's centroid loads fly together
+            constexpr int EPW = EP / kWaves;
+            double a[EPW];
+            const float* cr[EPW];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) a[j] += xv * (double)C[(size_t)min(e0 + j, E - 1) * d + k];
+            for (int j = 0; j < EPW; ++j) {
+                a[j] = 0.0;
+                cr[j] = C + (size_t)(e0 + min(wave + j * kWaves, nvalid - 1)) * d;  // clamped: extra results are dropped
+            }
+            if (VEC) {
+#pragma unroll 4
+                for (int k = 4 * lane; k < d; k += 256) {
+                    const v4f xv = *reinterpret_cast<const v4f*>(xr + k);
+                    v4f gv = {1.f, 1.f, 1.f, 1.f};
+                    if (use_gamma) gv = *reinterpret_cast<const v4f*>(gamma + k);
+                    const double x0 = ((double)xv.x - mu) * (double)gv.x, x1 = ((double)xv.y - mu) * (double)gv.y;
+                    const double x2 = ((double)xv.z - mu) * (double)gv.z, x3 = ((double)xv.w - mu) * (double)gv.w;
+#pragma unroll
+                    for (int j = 0; j < EPW; ++j) {
+                        const v4f cv = *reinterpret_cast<const v4f*>(cr[j] + k);
+                        a[j] += (x0 * (double)cv.x + x1 * (double)cv.y) + (x2 * (double)cv.z + x3 * (double)cv.w);
+                    }
+                }
+            } else {
+                for (int k = lane; k < d; k += 64) {
+                    const double xg = ((double)xr[k] - mu) * (use_gamma ? (double)gamma[k] : 1.0);
+#pragma unroll
+                    for (int j = 0; j < EPW; ++j) a[j] += xg * (double)cr[j][k];
+                }
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                a[j] = wave_sum(a[j]);
-                if (lane == 0) s_red[wave][j] = a[j];
+            for (int j = 0; j < EPW; ++j) {
+                const double sum = wave_sum(a[j]);
+                if (lane == 0 && wave + j * kWaves < nvalid) s_sc64[wave + j * kWaves] = sum;
             }
             __syncthreads();
             if (tid == 0) {
-                for (int j = 0; j < 8 && e0 + j < E; ++j) {
-                    double sc = rstd * ((s_red[0][j] + s_red[1][j]) + (s_red[2][j] + s_red[3][j]));
-                    if (bias != nullptr) sc += (double)bias[e0 + j];
+                for (int e = 0; e < nvalid; ++e) {  // ascending index, strict '>': lowest index wins ties
+                    double sc = rstd * s_sc64[e];
+                    if (bias != nullptr) sc += (double)bias[e0 + e];
                     if (sc > best) {
                         second = best;
                         best = sc;
-                        besti = e0 + j;
+                        besti = e0 + e;
                     } else if (sc > second) {
                         second = sc;
                     }
@@ -333,10 +402,15 @@ hipError_t launch_nblk(int T, int d, int E, const float* x, const float* c, cons
     const dim3 grid((T + kTokens - 1) / kTokens), block(kThreads);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(c) |
                            reinterpret_cast<uintptr_t>(gamma)) & 15) == 0;
-    if (d % 4 == 0 && aligned)
-        gate_top1_kernel<NBLK, true><<<grid, block, 0, stream>>>(T, d, E, x, c, gamma, norm_kind, bias, sel, coeff, stats);
-    else
-        gate_top1_kernel<NBLK, false><<<grid, block, 0, stream>>>(T, d, E, x, c, gamma, norm_kind, bias, sel, coeff, stats);
+    const bool vec = d % 4 == 0 && aligned;
+    const bool use_gamma = norm_kind != NORM_NONE && gamma != nullptr;
+#define INFMOE_GATE(V, G) \
+    gate_top1_kernel<NBLK, V, G><<<grid, block, 0, stream>>>(T, d, E, x, c, gamma, norm_kind, bias, sel, coeff, stats)
+    if (vec && use_gamma) INFMOE_GATE(true, true);
+    else if (vec) INFMOE_GATE(true, false);
+    else if (use_gamma) INFMOE_GATE(false, true);
+    else INFMOE_GATE(false, false);
+#undef INFMOE_GATE
     return hipGetLastError();
 }
 
