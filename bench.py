@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# benchmark scaled by what the same counters read for the row-copy kernels of known size
+# (profiles/c2_expert_gemm_grouped_kernel_stats.txt).  Counters cannot be read from inside a run.
+MEASURED_TRAFFIC_BYTES = {"c2": 5.70e9}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
@@ -179,7 +183,8 @@ def main():
     else:
         flops_per_launch = 2.0 * T * d * h
         roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
-                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": None,
+                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
                     "kernel": "expert_gemm_grouped_kernel (two launches per step: wi with ReLU, wo with residual)",
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
