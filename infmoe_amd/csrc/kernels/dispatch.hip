@@ -42,15 +42,22 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int*
 
 constexpr int kMaxSortedTiles = 1024;  // row tiles the scan orders by cost; beyond that they stay in expert order
 
-// `tiles` holds 2*max_tiles entries: the schedule first, then the raw list in expert order.
-// `sched` holds kSchedInts ints: [0] number of row tiles, [1 + x] first tile of XCD x (x = 0..8).
+// `tiles` holds 2*max_tiles entries (the second half is spare), `sched` kSchedInts ints:
+// [0] number of row tiles, [1 + x] first tile of XCD x (x = 0..8).
+// Everything the single workgroup touches more than once lives in LDS: a chain of dependent global
+// reads by one thread costs about a microsecond per link.
 __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, int* __restrict__ blockhist,
                                                         int* __restrict__ count, int* __restrict__ offset,
                                                         RowTile* __restrict__ tiles, int* __restrict__ sched,
                                                         int max_tiles, int xcd_cap, int tile_rows, int skinny_max) {
-    __shared__ int s_n;
-    __shared__ int s_cost[kMaxSortedTiles], s_order[kMaxSortedTiles];
-    __shared__ unsigned char s_bin[kMaxSortedTiles];
+    extern __shared__ int s_dyn[];  // [count E | offset E | first tile E]
+    int* s_count = s_dyn;
+    int* s_off = s_dyn + E;
+    int* s_tile0 = s_dyn + 2 * E;
+    __shared__ int s_n, s_total;
+    __shared__ RowTile s_raw[kMaxSortedTiles];
+    __shared__ int s_cost[kMaxSortedTiles];
+    __shared__ int s_sched[kSchedInts];
     for (int e = threadIdx.x; e < E; e += kThreads) {
         int run = 0;
         for (int b = 0; b < nblk; ++b) {
@@ -58,77 +65,81 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, 
             blockhist[(size_t)b * E + e] = run;  // tokens of e in earlier blocks
             run += c;
         }
+        s_count[e] = run;
         count[e] = run;
     }
     __syncthreads();
-    RowTile* raw = tiles ? tiles + max_tiles : nullptr;
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0) {  // exclusive prefixes of rows and of row tiles (LDS only)
         int off = 0, nt = 0;
         for (int e = 0; e < E; ++e) {
-            const int c = count[e];
-            offset[e] = off;
-            if (tiles != nullptr && c > skinny_max) {
-                for (int m0 = 0; m0 < c; m0 += tile_rows) {
-                    RowTile rt;
-                    rt.expert = e;
-                    rt.row0 = off + m0;
-                    rt.rows = min(tile_rows, c - m0);
-                    rt.pad = 0;
-                    raw[nt++] = rt;
-                }
-            }
+            const int c = s_count[e];
+            s_off[e] = off;
+            s_tile0[e] = nt;
+            if (c > skinny_max) nt += (c + tile_rows - 1) / tile_rows;
             off += c;
         }
-        offset[E] = off;  // == T (plugin/MoELayerPlugin.cc:351)
+        s_total = off;
         s_n = nt;
     }
     __syncthreads();
+    for (int e = threadIdx.x; e < E; e += kThreads) offset[e] = s_off[e];
+    if (threadIdx.x == 0) offset[E] = s_total;  // == T (plugin/MoELayerPlugin.cc:351)
     if (tiles == nullptr) return;
     const int n = s_n;
-    if (n > kMaxSortedTiles) {  // many tiles balance by themselves: equal contiguous shares
-        for (int j = threadIdx.x; j < n; j += kThreads) tiles[j] = raw[j];
+    const bool sorted = n <= kMaxSortedTiles;
+    for (int e = threadIdx.x; e < E; e += kThreads) {
+        const int c = s_count[e];
+        if (c <= skinny_max) continue;
+        int j = s_tile0[e];
+        for (int m0 = 0; m0 < c; m0 += tile_rows, ++j) {
+            RowTile rt;
+            rt.expert = e;
+            rt.row0 = s_off[e] + m0;
+            rt.rows = min(tile_rows, c - m0);
+            rt.pad = 0;
+            if (sorted)
+                s_raw[j] = rt;
+            else
+                tiles[j] = rt;  // many tiles balance by themselves: expert order, equal contiguous shares
+        }
+    }
+    if (!sorted) {
         if (threadIdx.x <= kXcdCount) sched[1 + threadIdx.x] = (int)(((long long)n * threadIdx.x) / kXcdCount);
         if (threadIdx.x == 0) sched[0] = n;
         return;
     }
-    // Longest-processing-time-first over the 8 XCDs: order the tiles by padded height (the cost of
-    // a tile), then give each to the least loaded XCD.  Inside an XCD the order stays descending,
-    // so the short tiles fill the tail.
-    for (int j = threadIdx.x; j < n; j += kThreads) s_cost[j] = (raw[j].rows + 15) >> 4;
+    __syncthreads();
+    // Balance the 8 XCDs: order the tiles by padded height (the cost of a tile) and deal them out in
+    // snake order (XCD 0..7, then 7..0, ...), which keeps the loads within one tile of each other and,
+    // unlike a greedy assignment, lets every tile compute its own place.  Inside an XCD the order
+    // stays descending, so the short tiles fill the tail.
+    for (int j = threadIdx.x; j < n; j += kThreads) s_cost[j] = (s_raw[j].rows + 15) >> 4;
+    __syncthreads();
+    const int full = n / kXcdCount, rem = n % kXcdCount;
+    auto share = [&](int x) {  // tiles of XCD x: one per full round plus its part of the last, partial round
+        const bool extra = (full & 1) == 0 ? x < rem : x >= kXcdCount - rem;
+        return full + (extra ? 1 : 0);
+    };
+    if (threadIdx.x == 0) {
+        int start = 0;
+        s_sched[0] = n;
+        for (int x = 0; x < kXcdCount; ++x) {
+            s_sched[1 + x] = start;
+            start += share(x);
+        }
+        s_sched[1 + kXcdCount] = start;
+    }
     __syncthreads();
     for (int j = threadIdx.x; j < n; j += kThreads) {
         const int cj = s_cost[j];
         int rank = 0;
         for (int i = 0; i < n; ++i) rank += (s_cost[i] > cj) || (s_cost[i] == cj && i < j);
-        s_order[rank] = j;
+        const int round = rank / kXcdCount, idx = rank % kXcdCount;
+        const int x = (round & 1) == 0 ? idx : kXcdCount - 1 - idx;
+        tiles[s_sched[1 + x] + round] = s_raw[j];
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int load[kXcdCount], cnt[kXcdCount];
-        for (int x = 0; x < kXcdCount; ++x) load[x] = 0, cnt[x] = 0;
-        for (int r = 0; r < n; ++r) {
-            const int j = s_order[r];
-            int best = -1;
-            for (int x = 0; x < kXcdCount; ++x)
-                if (cnt[x] < xcd_cap && (best < 0 || load[x] < load[best])) best = x;
-            if (best < 0) best = r % kXcdCount;  // cannot happen while 8 * xcd_cap >= n
-            s_bin[j] = (unsigned char)best;
-            load[best] += s_cost[j];
-            cnt[best]++;
-        }
-        int start = 0;
-        sched[0] = n;
-        for (int x = 0; x < kXcdCount; ++x) {
-            sched[1 + x] = start;
-            load[x] = start;  // reused as the fill cursor
-            start += cnt[x];
-        }
-        sched[1 + kXcdCount] = start;
-        for (int r = 0; r < n; ++r) {
-            const int j = s_order[r];
-            tiles[load[s_bin[j]]++] = raw[j];
-        }
-    }
+    if (threadIdx.x < 2 + kXcdCount) sched[threadIdx.x] = s_sched[threadIdx.x];
+    (void)xcd_cap;  // a share never exceeds ceil(n / 8), which is below the capacity the grid was sized for
 }
 
 __global__ __launch_bounds__(kThreads) void rank_kernel(int T, int E, const int* __restrict__ sel,
@@ -279,7 +290,7 @@ hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* coun
     const size_t lds = (size_t)E * sizeof(int);
     if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
     const int max_tiles = max_row_tiles(T, E, tile_rows);
-    scan_kernel<<<1, kThreads, 0, stream>>>(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles,
+    scan_kernel<<<1, kThreads, 3 * lds, stream>>>(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles,
                                             xcd_tile_capacity(max_tiles), tile_rows, skinny_max);
     if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);
     return hipGetLastError();

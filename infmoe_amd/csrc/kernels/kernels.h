@@ -17,9 +17,14 @@ constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/subla
 
 // ---- gating (replaces layernorm_gpu + cublasSgemm + expert_select_top1_kernel,
 //      plugin/MoELayerPlugin.cc:315-345)
+// Optional: folded_centroids [E][d] = centroids * gamma (device) and centroid_stats [2E] = per expert
+// the sum and the Euclidean norm of that product (device), both made by fold_centroids_host; with
+// them the kernel skips work that depends on the layer's parameters only.
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
-                            hipStream_t stream);
+                            hipStream_t stream, const float* folded_centroids = nullptr,
+                            const float* centroid_stats = nullptr);
+void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)
 // Row tile of the grouped expert GEMM: `rows` consecutive routed rows of one expert.

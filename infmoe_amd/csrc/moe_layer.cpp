@@ -185,6 +185,14 @@ Status MoELayer::initialize() {
         INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mLayernormGpu), sizeof(float) * d));
         INFMOE_HIP(hipMemcpy(mLayernormGpu, mParams.layernormWeight.data(), sizeof(float) * d, hipMemcpyHostToDevice));
     }
+    {   // what the gating kernel needs of (centroids, gamma) and would otherwise recompute per workgroup
+        std::vector<float> folded((size_t)E * d + 2 * (size_t)E);
+        const bool ln = mParams.flags.layernormOnInputBeforeScore;
+        fold_centroids_host(d, E, mParams.centroids.data(), ln ? mParams.layernormWeight.data() : nullptr, folded.data(),
+                            folded.data() + (size_t)E * d);
+        INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mFoldedGpu), sizeof(float) * folded.size()));
+        INFMOE_HIP(hipMemcpy(mFoldedGpu, folded.data(), sizeof(float) * folded.size(), hipMemcpyHostToDevice));
+    }
     const size_t routingInts = (size_t)2 * E + 1 + 4;
     INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mRoutingGpu), sizeof(int32_t) * routingInts));
     INFMOE_HIP(hipMemset(mRoutingGpu, 0, sizeof(int32_t) * routingInts));
@@ -217,6 +225,8 @@ Status MoELayer::terminate() {
     if (mCentroidsGpu) (void)hipFree(mCentroidsGpu);
     if (mLayernormGpu) (void)hipFree(mLayernormGpu);
     if (mScoreBiasGpu) (void)hipFree(mScoreBiasGpu);
+    if (mFoldedGpu) (void)hipFree(mFoldedGpu);
+    mFoldedGpu = nullptr;
     if (mRoutingGpu) (void)hipFree(mRoutingGpu);
     if (mRoutingHost) (void)hipHostFree(mRoutingHost);
     mCentroidsGpu = mLayernormGpu = mScoreBiasGpu = nullptr;
@@ -271,7 +281,8 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     INFMOE_HIP(launch_fill_i32(dStats, 4, 0, stream));
     const bool ln = mParams.flags.layernormOnInputBeforeScore;
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
-                                mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream));
+                                mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream, mFoldedGpu,
+                                mFoldedGpu + (size_t)E * d));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     const bool grouped = resident();

@@ -72,6 +72,7 @@ class MoELayer {
     float* mCentroidsGpu = nullptr;
     float* mLayernormGpu = nullptr;
     float* mScoreBiasGpu = nullptr;
+    float* mFoldedGpu = nullptr;      // centroids * gating gamma [E][d], then [sum E | norm E]
     int32_t* mRoutingGpu = nullptr;   // [count E | offset E+1 | stats 4]
     int32_t* mRoutingHost = nullptr;  // page-locked mirror
     hipStream_t mCopyStream = nullptr;
