@@ -344,12 +344,6 @@ size_t lds_bytes(int a_alloc_rows) {
     return (2 * (size_t)a_alloc_rows * LDK + 2 * (size_t)(GATED ? 2 : 1) * BN * LDK) * sizeof(float);
 }
 
-template <typename Kern>
-hipError_t allow_lds(Kern kern, size_t bytes) {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)bytes);
-}
-
 bool fast_path_ok(const GemmProblem& p) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B) |
                            reinterpret_cast<uintptr_t>(p.B1);
@@ -373,11 +367,11 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
         const size_t lds = lds_bytes<kBN, true>(a_alloc);
-        if ((err = allow_lds(expert_gemm_kernel<kBN, true>, lds_bytes<kBN, true>(kGemmTileRowsGated))) != hipSuccess) return err;
+        if ((err = allow_lds_once<expert_gemm_kernel<kBN, true>>(lds_bytes<kBN, true>(kGemmTileRowsGated))) != hipSuccess) return err;
         expert_gemm_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, rows, a_alloc);
     } else {
         const size_t lds = lds_bytes<kBN, false>(a_alloc);
-        if ((err = allow_lds(expert_gemm_kernel<kBN, false>, lds_bytes<kBN, false>(kGemmTileRows))) != hipSuccess) return err;
+        if ((err = allow_lds_once<expert_gemm_kernel<kBN, false>>(lds_bytes<kBN, false>(kGemmTileRows))) != hipSuccess) return err;
         expert_gemm_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, rows, a_alloc);
     }
     return hipGetLastError();
@@ -392,11 +386,11 @@ hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
         const size_t lds = lds_bytes<kBN, true>(kGemmTileRowsGated);
-        if ((err = allow_lds(expert_gemm_grouped_kernel<kBN, true>, lds)) != hipSuccess) return err;
+        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, true>>(lds)) != hipSuccess) return err;
         expert_gemm_grouped_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     } else {
         const size_t lds = lds_bytes<kBN, false>(kGemmTileRows);
-        if ((err = allow_lds(expert_gemm_grouped_kernel<kBN, false>, lds)) != hipSuccess) return err;
+        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, false>>(lds)) != hipSuccess) return err;
         expert_gemm_grouped_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     }
     return hipGetLastError();

@@ -568,8 +568,7 @@ hipError_t launch_nblk(int T, int d, int E, const float* x, const float* c, cons
 #define INFMOE_GATE(V, G, P)                                                                                       \
     do {                                                                                                           \
         const size_t lds = 2 * (size_t)(kTokens + 16 * NBLK + ((G) && !(P) ? 1 : 0)) * (KC + 4) * sizeof(float);   \
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(gate_top1_kernel<NBLK, V, G, P>),                  \
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                           \
+        err = allow_lds_once<gate_top1_kernel<NBLK, V, G, P>>(lds);                                                \
         if (err != hipSuccess) return err;                                                                         \
         gate_top1_kernel<NBLK, V, G, P><<<grid, block, lds, stream>>>(T, d, E, x, c, gamma, cf, cstats, norm_kind, \
                                                                       bias, sel, coeff, stats);                    \

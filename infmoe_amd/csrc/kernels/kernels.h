@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 
@@ -100,5 +101,21 @@ constexpr int kSkinnyMaxRows = 8;
 hipError_t launch_expert_skinny(const GemmProblem& p, int rows, hipStream_t stream);
 hipError_t launch_expert_skinny_grouped(const GemmProblem& p, size_t weight_stride, const int* count,
                                         const int* offset, int E, hipStream_t stream);
+
+// Kernels whose dynamic LDS exceeds 64 KB need the limit raised once per device.  Doing it on the
+// first launch only keeps later launches free of runtime calls other than the launch itself, so a
+// caller may capture them in a graph after one eager call.
+template <auto Kern>
+inline hipError_t allow_lds_once(size_t bytes) {
+    static std::atomic<uint64_t> done{0};
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (err == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return err;
+}
 
 }  // namespace infmoe

@@ -216,3 +216,34 @@ def test_enqueue_before_initialize_is_an_error(torch_cuda):
     with pytest.raises(capi.InfMoEError) as ei:
         plugin.forward(dev(torch_cuda, x.reshape(1, 8, 16)))
     assert ei.value.status == capi.ERR_STATE
+
+
+def test_layer_can_be_captured_in_a_graph_and_replayed(torch_cuda):
+    """The resident schedule makes no host wait and no allocation, so after one eager call it can be
+    captured; every replay, with eager work in between, must reproduce the eager result bit for bit."""
+    torch = torch_cuda
+    shape, E, d, h = (4, 64), 8, 128, 256
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, E, "cpm_2", seed=43)
+    xs = [dev(torch, np.roll(x, k, axis=0).reshape(4, 64, d)) for k in range(3)]
+    eager = [plugin.forward(v).clone() for v in xs]
+    dims = [4, 64, d]
+    wsb = torch.empty(plugin.workspace_size(dims), dtype=torch.uint8, device="cuda")
+    xin = xs[0].clone()
+    yout = torch.empty_like(xin)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plugin.enqueue(dims, xin.data_ptr(), yout.data_ptr(), wsb.data_ptr(), side.cuda_stream)  # warm
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plugin.enqueue(dims, xin.data_ptr(), yout.data_ptr(), wsb.data_ptr(), side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(2):
+        for k, v in enumerate(xs):
+            xin.copy_(v)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(yout, eager[k]), f"replay {rep}/{k} differs from the eager result"
+            assert torch.equal(plugin.forward(v), eager[k])  # eager work between replays
+    plugin.terminate()
