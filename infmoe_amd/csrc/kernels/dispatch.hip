@@ -25,9 +25,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
 constexpr int kPerThread = kCountBlockTokens / kThreads;
 
-__global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int* __restrict__ sel,
-                                                        int* __restrict__ blockhist) {
-    extern __shared__ int s_hist[];
+__device__ __forceinline__ void hist_body(int T, int E, const int* __restrict__ sel, int* __restrict__ blockhist,
+                                          int* s_hist) {
     for (int e = threadIdx.x; e < E; e += kThreads) s_hist[e] = 0;
     __syncthreads();
     const int base = blockIdx.x * kCountBlockTokens;
@@ -40,17 +39,23 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int*
     for (int e = threadIdx.x; e < E; e += kThreads) blockhist[(size_t)blockIdx.x * E + e] = s_hist[e];
 }
 
+__global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int* __restrict__ sel,
+                                                        int* __restrict__ blockhist) {
+    extern __shared__ int s_dyn[];
+    hist_body(T, E, sel, blockhist, s_dyn);
+}
+
 constexpr int kMaxSortedTiles = 1024;  // row tiles the scan orders by cost; beyond that they stay in expert order
 
 // `tiles` holds 2*max_tiles entries (the second half is spare), `sched` kSchedInts ints:
 // [0] number of row tiles, [1 + x] first tile of XCD x (x = 0..8).
 // Everything the single workgroup touches more than once lives in LDS: a chain of dependent global
 // reads by one thread costs about a microsecond per link.
-__global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, int* __restrict__ blockhist,
-                                                        int* __restrict__ count, int* __restrict__ offset,
-                                                        RowTile* __restrict__ tiles, int* __restrict__ sched,
-                                                        int max_tiles, int xcd_cap, int tile_rows, int skinny_max) {
-    extern __shared__ int s_dyn[];  // [count E | offset E | first tile E]
+__device__ __forceinline__ void scan_body(int T, int E, int nblk, int* __restrict__ blockhist,
+                                          int* __restrict__ count, int* __restrict__ offset,
+                                          RowTile* __restrict__ tiles, int* __restrict__ sched, int max_tiles,
+                                          int xcd_cap, int tile_rows, int skinny_max, int* s_dyn) {
+    // s_dyn: [count E | offset E | first tile E]
     int* s_count = s_dyn;
     int* s_off = s_dyn + E;
     int* s_tile0 = s_dyn + 2 * E;
@@ -140,13 +145,22 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, 
     }
     if (threadIdx.x < 2 + kXcdCount) sched[threadIdx.x] = s_sched[threadIdx.x];
     (void)xcd_cap;  // a share never exceeds ceil(n / 8), which is below the capacity the grid was sized for
+    (void)T;
+    (void)max_tiles;
 }
 
-__global__ __launch_bounds__(kThreads) void rank_kernel(int T, int E, const int* __restrict__ sel,
-                                                        const int* __restrict__ blockbase,
-                                                        const int* __restrict__ offset, int* __restrict__ pos,
-                                                        int* __restrict__ row_expert) {
-    extern __shared__ int s_run[];  // tokens of each expert already ranked in this block
+__global__ __launch_bounds__(kThreads) void scan_kernel(int T, int E, int nblk, int* __restrict__ blockhist,
+                                                        int* __restrict__ count, int* __restrict__ offset,
+                                                        RowTile* __restrict__ tiles, int* __restrict__ sched,
+                                                        int max_tiles, int xcd_cap, int tile_rows, int skinny_max) {
+    extern __shared__ int s_dyn[];
+    scan_body(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles, xcd_cap, tile_rows, skinny_max, s_dyn);
+}
+
+__device__ __forceinline__ void rank_body(int T, int E, const int* __restrict__ sel,
+                                          const int* __restrict__ blockbase, const int* __restrict__ offset,
+                                          int* __restrict__ pos, int* __restrict__ row_expert, int* s_run) {
+    // s_run: tokens of each expert already ranked in this block
     for (int e = threadIdx.x; e < E; e += kThreads) s_run[e] = offset[e] + blockbase[(size_t)blockIdx.x * E + e];
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -183,6 +197,32 @@ __global__ __launch_bounds__(kThreads) void rank_kernel(int T, int E, const int*
             __syncthreads();
         }
     }
+}
+
+__global__ __launch_bounds__(kThreads) void rank_kernel(int T, int E, const int* __restrict__ sel,
+                                                        const int* __restrict__ blockbase,
+                                                        const int* __restrict__ offset, int* __restrict__ pos,
+                                                        int* __restrict__ row_expert) {
+    extern __shared__ int s_dyn[];
+    rank_body(T, E, sel, blockbase, offset, pos, row_expert, s_dyn);
+}
+
+// Up to kCountBlockTokens tokens (decode shapes): the three steps in one launch of one workgroup.
+// What one step writes to global memory is read by the next after a barrier of the same workgroup.
+__global__ __launch_bounds__(kThreads) void count_small_kernel(int T, int E, const int* __restrict__ sel,
+                                                               int* __restrict__ blockhist, int* __restrict__ pos,
+                                                               int* __restrict__ count, int* __restrict__ offset,
+                                                               RowTile* __restrict__ tiles, int* __restrict__ sched,
+                                                               int max_tiles, int xcd_cap, int tile_rows,
+                                                               int skinny_max, int* __restrict__ row_expert) {
+    extern __shared__ int s_dyn[];
+    hist_body(T, E, sel, blockhist, s_dyn);
+    __threadfence_block();
+    __syncthreads();
+    scan_body(T, E, 1, blockhist, count, offset, tiles, sched, max_tiles, xcd_cap, tile_rows, skinny_max, s_dyn);
+    __threadfence_block();
+    __syncthreads();
+    rank_body(T, E, sel, blockhist, offset, pos, row_expert, s_dyn);
 }
 
 // ---- row copies: one wave per row, 16-byte accesses when the row length allows
@@ -288,8 +328,14 @@ hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* coun
     const int nblk = (T + kCountBlockTokens - 1) / kCountBlockTokens;
     int* blockhist = static_cast<int*>(scratch);
     const size_t lds = (size_t)E * sizeof(int);
-    if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
     const int max_tiles = max_row_tiles(T, E, tile_rows);
+    if (nblk == 1) {
+        count_small_kernel<<<1, kThreads, 3 * lds, stream>>>(T, E, sel, blockhist, pos, count, offset, tiles, sched,
+                                                             max_tiles, xcd_tile_capacity(max_tiles), tile_rows,
+                                                             skinny_max, row_expert);
+        return hipGetLastError();
+    }
+    if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
     scan_kernel<<<1, kThreads, 3 * lds, stream>>>(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles,
                                             xcd_tile_capacity(max_tiles), tile_rows, skinny_max);
     if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);
