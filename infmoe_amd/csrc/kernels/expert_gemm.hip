@@ -36,6 +36,7 @@
 // in one XCD's L2.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <type_traits>
 
 #include "kernels.h"
@@ -46,8 +47,7 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 32;            // k floats per pipeline step
-constexpr int LDK = BK + 4;       // padded LDS row (floats)
+constexpr int kMaxMb64 = 10;      // tallest tile (in 16-row units) that takes 64-float K steps: 160 rows
 constexpr int kThreads = 256;     // 4 waves
 
 __device__ __forceinline__ float gelu_dot(float a, float b) {
@@ -66,7 +66,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // One output tile: `rows` (<= 16*NMB) rows of A against BN rows of B (and of B1 when GATED).
-template <int NMB, int BN, bool GATED>
+// BK: floats of K per pipeline step (32 or 64).
+template <int NMB, int BN, bool GATED, int BK>
 __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const float* __restrict__ R,
                                           float* __restrict__ C, int rows, const float* __restrict__ B0,
                                           const float* __restrict__ B1, int n0, int N, int K, int epilogue,
@@ -75,9 +76,11 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     constexpr int NB = GATED ? 2 : 1;         // weight matrices
     constexpr int N32 = NMB / 2;              // 32-row blocks (v_mfma_f32_32x32x2_f32)
     constexpr bool T16 = (NMB & 1) != 0;      // one trailing 16-row block (v_mfma_f32_16x16x4_f32)
+    constexpr int LDK = BK + 4;               // padded LDS row (floats)
+    constexpr int KH = BK / 32;               // 32-float halves of a step's row
     constexpr int A_ROWS = NMB * 16;
-    constexpr int A_LOADS = (A_ROWS + 31) / 32;  // float4 per thread per step: one per 32-row slab
-    constexpr int B_LOADS = BN / 32;
+    constexpr int A_LOADS = ((A_ROWS + 31) / 32) * KH;  // float4 per thread per step: KH per 32-row slab
+    constexpr int B_LOADS = (BN / 32) * KH;
     constexpr int NV = A_LOADS + NB * B_LOADS;   // global loads (and LDS writes) per thread per step
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -110,16 +113,16 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     if (GATED) b_base[NB - 1] = reinterpret_cast<const char*>(B1 + (size_t)n0 * K);
     unsigned a_off[A_LOADS], b_off[B_LOADS];
 #pragma unroll
-    for (int p = 0; p < A_LOADS; ++p)
-        a_off[p] = ((unsigned)min(p * 32 + ld_row, rows - 1) * (unsigned)K + 4u * ld_c4) * 4u;
+    for (int p = 0; p < A_LOADS; ++p)  // item p: slab p / KH, half p % KH
+        a_off[p] = ((unsigned)min((p / KH) * 32 + ld_row, rows - 1) * (unsigned)K + 32u * (p % KH) + 4u * ld_c4) * 4u;
 #pragma unroll
     for (int p = 0; p < B_LOADS; ++p)
-        b_off[p] = ((unsigned)min(p * 32 + ld_row, N - 1 - n0) * (unsigned)K + 4u * ld_c4) * 4u;
+        b_off[p] = ((unsigned)min((p / KH) * 32 + ld_row, N - 1 - n0) * (unsigned)K + 32u * (p % KH) + 4u * ld_c4) * 4u;
 
     // Two register sets: global loads run two K steps ahead of the matrix core, which covers the
     // latency of an HBM miss (every weight load is one) with two steps of MFMA work.
     v4f ra[2][A_LOADS], rb[2][NB][B_LOADS];
-    // item L of the global loads of the step starting at k0 (K % 32 == 0 on this path), into set P
+    // item L of the global loads of the step starting at k0 (K % BK == 0 on this path), into set P
     auto gload = [&](auto setc, auto lc, int k0) {
         constexpr int P = decltype(setc)::value, L = decltype(lc)::value;
         if constexpr (L < A_LOADS) {
@@ -133,10 +136,11 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     auto lstore = [&](auto setc, auto lc, auto bufc) {
         constexpr int P = decltype(setc)::value, L = decltype(lc)::value, BUF = decltype(bufc)::value;
         if constexpr (L < A_LOADS) {
-            *reinterpret_cast<v4f*>(As + BUF * a_buf + (L * 32 + ld_row) * LDK + 4 * ld_c4) = ra[P][L];
+            *reinterpret_cast<v4f*>(As + BUF * a_buf + ((L / KH) * 32 + ld_row) * LDK + 32 * (L % KH) + 4 * ld_c4) = ra[P][L];
         } else {
             constexpr int M = (L - A_LOADS) / B_LOADS, Q = (L - A_LOADS) % B_LOADS;
-            *reinterpret_cast<v4f*>(Bs + BUF * b_buf + (M * BN + Q * 32 + ld_row) * LDK + 4 * ld_c4) = rb[P][M][Q];
+            *reinterpret_cast<v4f*>(Bs + BUF * b_buf + (M * BN + (Q / KH) * 32 + ld_row) * LDK + 32 * (Q % KH) + 4 * ld_c4) =
+                rb[P][M][Q];
         }
     };
 
@@ -170,7 +174,8 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     //   * every slot group carries the LDS operand reads of the next k group.
     // The loop over steps is unrolled by two so that P, and with it every LDS address offset and
     // register index, is a compile-time constant.
-    constexpr int S32 = N32 > 0 ? 16 : 0, S16 = T16 ? 8 : 0, S = S32 + S16, SV = S / 2;
+    constexpr int G32 = BK / 8, G16 = BK / 16;  // k groups of a step
+    constexpr int S32 = N32 > 0 ? 4 * G32 : 0, S16 = T16 ? 4 * G16 : 0, S = S32 + S16, SV = S / 2;
     constexpr int R32 = NB + N32, R16 = 1 + 2 * NB;
     const int nk = K / BK;
     auto step = [&](auto setc, int s) {
@@ -191,11 +196,11 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
                     [&](auto lc) { lstore(cur, lc, other); });
             if constexpr (t < S32) {
                 constexpr int g = t / 4, j = t % 4;
-                if constexpr (g < 3 && j < 3)  // a third of the next group's operands per slot
+                if constexpr (g < G32 - 1 && j < 3)  // a third of the next group's operands per slot
                     static_for<0, R32>([&](auto qc) {
                         if constexpr (decltype(qc)::value % 3 == j) read32(cur, std::integral_constant<int, g + 1>{}, qc);
                     });
-                if constexpr (g == 3 && j < 3 && T16)
+                if constexpr (g == G32 - 1 && j < 3 && T16)
                     static_for<0, R16>([&](auto qc) {
                         if constexpr (decltype(qc)::value % 3 == j) read16(cur, std::integral_constant<int, 0>{}, qc);
                     });
@@ -207,9 +212,9 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
                                                                              acc32[m][mb], 0, 0, 0);
             } else {
                 constexpr int g = (t - S32) / 4, j = (t - S32) % 4;
-                if constexpr (g == 0 && j < 3)
+                if constexpr (g < G16 - 1 && j < 3)
                     static_for<0, R16>([&](auto qc) {
-                        if constexpr (decltype(qc)::value % 3 == j) read16(cur, std::integral_constant<int, 1>{}, qc);
+                        if constexpr (decltype(qc)::value % 3 == j) read16(cur, std::integral_constant<int, g + 1>{}, qc);
                     });
 #pragma unroll
                 for (int m = 0; m < NB; ++m)
@@ -269,10 +274,21 @@ __device__ __forceinline__ void gemm_dispatch(int nmb, const float* A, const flo
                                               float* smem, int a_alloc_rows) {
     // the gated form keeps two accumulator sets, so its tiles are half as tall
     constexpr int kMaxMb = (GATED ? kGemmTileRowsGated : kGemmTileRows) / 16;
+    // Tiles of up to 160 rows take K in steps of 64 floats (half as many barriers per flop); the LDS
+    // cannot hold two such stages of a taller tile or of two weight matrices, which take steps of 32.
+    const bool wide = !GATED && (K & 63) == 0;
 #define INFMOE_CASE(n)                                                                                       \
     case n:                                                                                                  \
-        if constexpr (n <= kMaxMb)                                                                           \
-            gemm_tile<n, BN, GATED>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);          \
+        if constexpr (n <= kMaxMb) {                                                                         \
+            if constexpr (!GATED && n <= kMaxMb64) {                                                         \
+                if (wide) {                                                                                  \
+                    gemm_tile<n, BN, GATED, 64>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem,             \
+                                                min(a_alloc_rows, 16 * kMaxMb64));                           \
+                    break;                                                                                   \
+                }                                                                                            \
+            }                                                                                                \
+            gemm_tile<n, BN, GATED, 32>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);      \
+        }                                                                                                    \
         break;
     switch (nmb) {
         INFMOE_CASE(1) INFMOE_CASE(2) INFMOE_CASE(3) INFMOE_CASE(4) INFMOE_CASE(5) INFMOE_CASE(6) INFMOE_CASE(7)
@@ -339,18 +355,26 @@ __global__ void expert_gemm_generic_kernel(GemmProblem p, int rows) {
     p.C[idx] = s0;
 }
 
+// LDS the kernel may touch for tiles of up to a_alloc_rows rows: the larger of the two step widths.
 template <int BN, bool GATED>
-size_t lds_bytes(int a_alloc_rows) {
-    return (2 * (size_t)a_alloc_rows * LDK + 2 * (size_t)(GATED ? 2 : 1) * BN * LDK) * sizeof(float);
+size_t lds_bytes(int a_alloc_rows, int K) {
+    const size_t nb = GATED ? 2 : 1;
+    size_t bytes = (2 * (size_t)a_alloc_rows * 36 + 2 * nb * BN * 36) * sizeof(float);
+    if (!GATED && K % 64 == 0) {
+        const size_t rows64 = (size_t)std::min(a_alloc_rows, 16 * kMaxMb64);
+        bytes = std::max(bytes, (2 * rows64 * 68 + 2 * nb * BN * 68) * sizeof(float));
+    }
+    return bytes;
 }
 
 bool fast_path_ok(const GemmProblem& p) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B) |
                            reinterpret_cast<uintptr_t>(p.B1);
-    return p.K % BK == 0 && (bits & 15) == 0;
+    return p.K % 32 == 0 && (bits & 15) == 0;
 }
 
 constexpr int kBN = 128;
+constexpr size_t kLdsPerCu = 160 * 1024;  // the limit is raised once, to all there is; launches ask for what they use
 
 }  // namespace
 
@@ -366,12 +390,12 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
     const dim3 grid((p.N + kBN - 1) / kBN, (rows + tile - 1) / tile);
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
-        const size_t lds = lds_bytes<kBN, true>(a_alloc);
-        if ((err = allow_lds_once<expert_gemm_kernel<kBN, true>>(lds_bytes<kBN, true>(kGemmTileRowsGated))) != hipSuccess) return err;
+        const size_t lds = lds_bytes<kBN, true>(a_alloc, p.K);
+        if ((err = allow_lds_once<expert_gemm_kernel<kBN, true>>(kLdsPerCu)) != hipSuccess) return err;
         expert_gemm_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, rows, a_alloc);
     } else {
-        const size_t lds = lds_bytes<kBN, false>(a_alloc);
-        if ((err = allow_lds_once<expert_gemm_kernel<kBN, false>>(lds_bytes<kBN, false>(kGemmTileRows))) != hipSuccess) return err;
+        const size_t lds = lds_bytes<kBN, false>(a_alloc, p.K);
+        if ((err = allow_lds_once<expert_gemm_kernel<kBN, false>>(kLdsPerCu)) != hipSuccess) return err;
         expert_gemm_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, rows, a_alloc);
     }
     return hipGetLastError();
@@ -385,12 +409,12 @@ hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride
     const dim3 grid((unsigned)kXcdCount * (unsigned)xcd_tile_capacity(max_tiles) * (unsigned)n_col_tiles);
     hipError_t err;
     if (p.epilogue == EPI_GATED_GELU) {
-        const size_t lds = lds_bytes<kBN, true>(kGemmTileRowsGated);
-        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, true>>(lds)) != hipSuccess) return err;
+        const size_t lds = lds_bytes<kBN, true>(kGemmTileRowsGated, p.K);
+        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, true>>(kLdsPerCu)) != hipSuccess) return err;
         expert_gemm_grouped_kernel<kBN, true><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     } else {
-        const size_t lds = lds_bytes<kBN, false>(kGemmTileRows);
-        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, false>>(lds)) != hipSuccess) return err;
+        const size_t lds = lds_bytes<kBN, false>(kGemmTileRows, p.K);
+        if ((err = allow_lds_once<expert_gemm_grouped_kernel<kBN, false>>(kLdsPerCu)) != hipSuccess) return err;
         expert_gemm_grouped_kernel<kBN, false><<<grid, kThreads, lds, stream>>>(p, weight_stride, tiles, sched, n_col_tiles);
     }
     return hipGetLastError();
