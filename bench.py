@@ -27,8 +27,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # benchmark scaled by what the same counters read for the row-copy kernels of known size
-# (profiles/c2_expert_gemm_grouped_kernel_stats.txt).  Counters cannot be read from inside a run.
-MEASURED_TRAFFIC_BYTES = {"c2": 5.70e9}
+# (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt).  Counters cannot be read from inside a run.
+MEASURED_TRAFFIC_BYTES = {"c2": 5.70e9, "c5": 4.04e9}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
@@ -177,7 +177,7 @@ def main():
     elif few_rows:
         bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
         roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": None,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
                     "kernel": "expert_skinny_kernel (two launches per step: wi with ReLU, wo with residual)",
                     "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     else:
