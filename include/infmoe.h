@@ -172,10 +172,15 @@ enum { INFMOE_FFN_RELU = 0, INFMOE_FFN_GATED_GELU = 1 };
  * x [T][d]; centroids [E][d]; gamma [d] or NULL (norm_kind NONE); score_bias [E] or NULL;
  * sel int32 [T]; coeff float [T] (the winning score); stats int32[3] as infmoe_last_routing
  * (accumulated with atomics: zero it first) or NULL.
+ * `scratch`: NULL, or infmoe_gate_top1_scratch_bytes(T,d,E) bytes (may be 0) of device memory (16-byte aligned,
+ * any contents): with it a call with few tokens spreads each token group's embedding dimension
+ * over several workgroups, which the reference's cuBLAS call does inside the library.  The result
+ * does not depend on it beyond FP32 rounding of the scores.
  */
+size_t infmoe_gate_top1_scratch_bytes(int32_t T, int32_t d, int32_t E);
 int32_t infmoe_gate_top1(int32_t T, int32_t d, int32_t E, const float* x, const float* centroids, const float* gamma,
                          int32_t norm_kind, const float* score_bias, int32_t* sel, float* coeff, int32_t* stats,
-                         void* hip_stream);
+                         void* scratch, void* hip_stream);
 
 /*
  * Replaces moe_expert_count (plugin/cuda/moe.cu:161-212), on the device and without a host

@@ -55,7 +55,8 @@ PROTOTYPES = {
     "infmoe_last_error": (C.c_char_p, []),
     "infmoe_plugin_name": (C.c_char_p, []),
     "infmoe_plugin_version": (C.c_char_p, []),
-    "infmoe_gate_top1": (_i32, [_i32, _i32, _i32, _pf, _pf, _pf, _i32, _pf, _vp, _pf, _vp, _vp]),
+    "infmoe_gate_top1_scratch_bytes": (_sz, [_i32, _i32, _i32]),
+    "infmoe_gate_top1": (_i32, [_i32, _i32, _i32, _pf, _pf, _pf, _i32, _pf, _vp, _pf, _vp, _vp, _vp]),
     "infmoe_expert_count_scratch_bytes": (_sz, [_i32, _i32]),
     "infmoe_expert_count": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "infmoe_expert_scatter": (_i32, [_i32, _i32, _pf, _pf, _vp, _pf, _pf, _vp]),

@@ -235,16 +235,22 @@ const char* infmoe_plugin_version(void) { return "1"; }
 #define INFMOE_NEED(cond, msg) \
     if (!(cond)) return fail(INFMOE_ERR_INVALID_ARGUMENT, msg)
 
+size_t infmoe_gate_top1_scratch_bytes(int32_t T, int32_t d, int32_t E) {
+    return sizeof(float) * gate_scratch_floats(T < 0 ? 0 : T, d < 1 ? 1 : d, E < 1 ? 1 : E);
+}
+
 int32_t infmoe_gate_top1(int32_t T, int32_t d, int32_t E, const float* x, const float* centroids, const float* gamma,
                          int32_t norm_kind, const float* score_bias, int32_t* sel, float* coeff, int32_t* stats,
-                         void* hip_stream) {
+                         void* scratch, void* hip_stream) {
     return guarded([&]() -> int32_t {
         INFMOE_NEED(T >= 0 && d > 0 && E > 0, "gate_top1: bad sizes");
         INFMOE_NEED(T == 0 || (x && centroids && sel && coeff), "gate_top1: null pointer");
         INFMOE_NEED(norm_kind >= NORM_NONE && norm_kind <= NORM_CENTERED, "gate_top1: bad norm_kind");
         INFMOE_NEED(norm_kind == NORM_NONE || gamma != nullptr, "gate_top1: norm needs gamma");
-        INFMOE_HIP(launch_gate_top1(T, d, E, x, centroids, gamma, norm_kind, score_bias, sel, coeff, stats,
-                                    static_cast<hipStream_t>(hip_stream)));
+        INFMOE_NEED((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "gate_top1: scratch must be 16-byte aligned");
+        hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+        INFMOE_HIP(launch_gate_top1(T, d, E, x, centroids, gamma, norm_kind, score_bias, sel, coeff, stats, stream, nullptr,
+                                    nullptr, static_cast<float*>(scratch), scratch ? gate_scratch_floats(T, d, E) : 0));
         return INFMOE_OK;
     });
 }

@@ -4,17 +4,26 @@
 // plugin/cuda/ops/layernorm.cu:136-188, plugin/cuda/moe.cu:13-76) and removes the
 // normalised-input and score-matrix round trips through memory.
 //
-// Work split: one workgroup (4 waves) owns 16 tokens and walks the embedding dimension in chunks
-// that are staged through LDS with row-contiguous global loads; each wave takes a quarter of every
-// chunk and runs v_mfma_f32_16x16x4_f32 with the tokens as the A rows and up to 128 experts
-// (8 column blocks) as the B columns.  The row
-// statistics of the norm are accumulated from the same registers that feed the matrix core,
-// and the norm is applied to the 16xE score tile instead of to the 16xd input:
+// Work split: one workgroup (4 waves) owns 16 or 64 tokens and a slice of the embedding dimension,
+// which it walks in chunks that are staged through LDS with row-contiguous global loads; each wave
+// takes a quarter of every chunk and runs v_mfma_f32_16x16x4_f32 with the tokens as the A rows and
+// up to 128 experts (8 column blocks) as the B columns.  The row statistics of the norm are
+// accumulated from the same registers that feed the matrix core, and the norm is applied to the
+// score tile instead of to the input:
 //     rms:      score = rstd * sum_k x_k g_k c_ek
 //     centered: score = rstd * (sum_k x_k g_k c_ek - mu * sum_k g_k c_ek)
-// Partial tiles of the 4 waves meet in LDS, then each wave reduces 4 tokens to
+// Partial tiles of the 4 waves meet in LDS, then 16 lanes reduce one token to
 // (best, index, runner-up) with the reference's tie rule (lowest index wins,
 // plugin/cuda/moe.cu:62-68).
+//
+// A compute unit can keep only about its first-level cache's worth of loads in flight, and every
+// workgroup reads all centroids, so what bounds the kernel is the traffic through that cache per
+// token: 64-token workgroups read a quarter of the centroid bytes per token that 16-token ones do.
+// To still fill the chip when there are few tokens, the embedding dimension is split over up to
+// 16 workgroups per token group; each writes its partial dot products and row sums to scratch
+// memory, and a second launch of the kernel adds them in slice order and does the selection.  (A
+// single launch in which the last workgroup to arrive combines the partial sums needs device-wide
+// fences, and those cost more here - about 8 us each with the chip busy - than the second launch.)
 //
 // FP32 accumulation over d terms cannot order two scores closer than its own rounding error,
 // so a token whose top-2 gap is below a Cauchy-Schwarz error bound is re-scored by the whole
@@ -24,6 +33,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cfloat>
+#include <algorithm>
 #include <cmath>
 #include <type_traits>
 
@@ -34,10 +44,43 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kTokens = 16;   // tokens per workgroup (MFMA M)
-constexpr int kWaves = 4;     // waves per workgroup; each takes a quarter of every staged K chunk
+constexpr int kWaves = 4;  // waves per workgroup; each takes a quarter of every staged K chunk
 constexpr int kThreads = 64 * kWaves;
-constexpr int kMaxCand = 4;   // near-tied experts the quick float64 re-scoring handles
+constexpr int kMaxCand = 4;          // near-tied experts the quick float64 re-scoring handles
+constexpr int kMaxSlices = 16;       // most workgroups that share one token group's embedding dimension
+constexpr int kTargetGroups = 256;   // workgroups wanted per launch: one per compute unit
+
+enum GateMode : int {
+    GATE_WHOLE = 0,    // one launch: scores, selection
+    GATE_SLICES = 1,   // first of two launches: partial scores of one slice of the embedding dimension
+    GATE_COMBINE = 2,  // second launch: add the slices' partial scores, selection
+};
+
+// Floats of K staged per step, by tile height (token rows + expert rows + gamma row): two buffers
+// of rows x (KC + 4) floats stay below 106 KB.
+constexpr int gate_kc(int nblk, int mb) {
+    const int rows = 16 * mb + 16 * nblk + 1;
+    return rows <= 49 ? 256 : (rows <= 97 ? 128 : 64);
+}
+
+struct GateArgs {
+    int T, d, E;
+    const float* X;
+    const float* C;
+    const float* gamma;
+    const float* Cf;      // centroids * gamma, or null
+    const float* cstats;  // [2E] sum and norm of the rows of Cf, or null
+    int norm_kind;
+    const float* bias;
+    int* sel;
+    float* coeff;
+    int* stats;
+    int mode;       // GateMode
+    int slices;     // workgroups per token group
+    int steps_per;  // K chunks per slice
+    float* partials;  // [slices][T][E + 2]: dot products, row sum, row sum of squares
+    float* gpart;     // [groups][slices][2E]: sum and sum of squares of the folded centroid slice
+};
 
 // Four floats of a row starting at k.  With VEC (d % 4 == 0, 16-byte aligned rows) the load is
 // unconditional: a k beyond the row is clamped to the last float4 and the caller discards the value
@@ -63,42 +106,54 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 // NBLK: 16-expert column blocks handled per pass (experts per pass = 16*NBLK).
+// MB: 16-token row blocks per workgroup.  With MB = 1 the four waves split every K chunk and their
+// partial tiles meet in LDS; with MB = 4 each wave owns 16 tokens and walks the whole chunk.
 // PRE: the caller supplies the centroids already multiplied by gamma (Cf) and, per expert, the sum
 // and the Euclidean norm of that product (cstats[0..E) and cstats[E..2E)): they depend on the layer's
 // parameters only, so the layer computes them once instead of every workgroup of every call.
-template <int NBLK, bool VEC, bool GAMMA, bool PRE>
-__global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E, const float* __restrict__ X,
-                                                             const float* __restrict__ C,
-                                                             const float* __restrict__ gamma,
-                                                             const float* __restrict__ Cf,
-                                                             const float* __restrict__ cstats, int norm_kind,
-                                                             const float* __restrict__ bias, int* __restrict__ sel,
-                                                             float* __restrict__ coeff, int* __restrict__ stats) {
+template <int NBLK, int MB, bool VEC, bool GAMMA, bool PRE>
+__global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg) {
     constexpr int EP = 16 * NBLK;
-    __shared__ float s_part[kWaves][kTokens][EP + 1];
-    __shared__ float s_score[kTokens][EP + 1];
-    __shared__ float s_s1[kWaves][kTokens], s_s2[kWaves][kTokens];
+    constexpr int TM = 16 * MB;
+    constexpr bool SPLITK = MB == 1;  // the waves split K (and meet in s_part) rather than the tokens
+    __shared__ float s_score[TM][EP + 1];
+    __shared__ float s_part[SPLITK ? kWaves : 1][SPLITK ? 16 : 1][SPLITK ? EP + 1 : 1];
+    __shared__ float s_s1[kWaves][16], s_s2[kWaves][16];
     __shared__ float s_g1[kWaves][EP], s_g2[kWaves][EP];
-    __shared__ float s_mu[kTokens], s_rstd[kTokens], s_xnorm[kTokens];
+    __shared__ float s_a1[TM], s_a2[TM];
+    __shared__ float s_mu[TM], s_rstd[TM], s_xnorm[TM];
     __shared__ float s_G[EP], s_cn[EP];
-    __shared__ float s_best[kTokens], s_second[kTokens], s_cnmax;
-    __shared__ int s_besti[kTokens], s_rescue[kTokens];
+    __shared__ float s_best[TM], s_second[TM], s_thr[TM], s_cnmax;
+    __shared__ int s_besti[TM], s_rescue[TM];
     __shared__ double s_red[kWaves][2];
     __shared__ double s_sc64[EP];
     __shared__ double s_bcast[2];
-    __shared__ float s_thr[kTokens];
     __shared__ int s_cand[kMaxCand], s_ncand;
     __shared__ double s_red2[kWaves][2 + 2 * kMaxCand];
+
+    const int T = arg.T, d = arg.d, E = arg.E, norm_kind = arg.norm_kind;
+    const float* __restrict__ X = arg.X;
+    const float* __restrict__ C = arg.C;
+    const float* __restrict__ gamma = arg.gamma;
+    const float* __restrict__ bias = arg.bias;
+    int* __restrict__ sel = arg.sel;
+    float* __restrict__ coeff = arg.coeff;
+    int* __restrict__ stats = arg.stats;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int i = lane & 15;   // A row (token) / B column (expert) this lane feeds
     const int kq = lane >> 4;  // which float4 of the 16-float chunk this lane feeds
-    const int t0 = blockIdx.x * kTokens;
     constexpr bool use_gamma = GAMMA;  // the norm's gamma is folded into the centroids as they are loaded
 
-    if (tid < kTokens) {
+    // Token group g, slice j of the embedding dimension.
+    const int S = arg.slices, mode = arg.mode;
+    const int g = mode == GATE_SLICES ? blockIdx.x / S : blockIdx.x;
+    const int j = mode == GATE_SLICES ? blockIdx.x % S : 0;
+    const int t0 = g * TM;
+
+    if (tid < TM) {
         s_best[tid] = -FLT_MAX;  // plugin/cuda/moe.cu:26-27
         s_second[tid] = -FLT_MAX;
         s_besti[tid] = -1;
@@ -106,136 +161,27 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
     }
     if (tid == 0) s_cnmax = 0.f;
 
-    // Staging tile in LDS, two buffers of ROWS x (KC + 4) floats: 16 token rows, EP centroid rows and
+    // Staging tile in LDS, two buffers of ROWS x (KC + 4) floats: the token rows, EP centroid rows and
     // (with a norm) the gamma row, KC floats of K at a time.  Every wave-wide global load reads whole
     // 512-byte or 1-KB stretches of one or two rows, which is what DRAM serves best; the MFMA operand
     // layout (a lane needs 16 bytes of "its" row) is produced by the LDS reads, not by the global loads.
-    constexpr int KC = NBLK <= 2 ? 256 : (NBLK == 4 ? 128 : 64);
+    constexpr int KC = gate_kc(NBLK, MB);
     constexpr int KC4 = KC / 4, LD = KC + 4;
     constexpr bool GROW = GAMMA && !PRE;  // stage a gamma row and fold it into the centroids here
-    constexpr int ROWS = kTokens + EP + (GROW ? 1 : 0);
+    constexpr int ROWS = TM + EP + (GROW ? 1 : 0);
     constexpr int NL = (ROWS * KC4 + kThreads - 1) / kThreads;  // 16-byte loads per thread per step
     extern __shared__ __align__(16) float s_tile[];
     const int nsteps = (d + KC - 1) / KC;
+    const int s_begin = j * arg.steps_per;
+    const int nst = min(nsteps - s_begin, arg.steps_per);  // >= 1 by the launcher's choice of slices
+    const int k_lo = s_begin * KC, k_hi = min(d, (s_begin + nst) * KC);
+    const int W = E + 2;  // floats per token and slice in `partials`
 
-    for (int e0 = 0; e0 < E; e0 += EP) {
-        v4f acc[NBLK];
-        float gs[NBLK], cn[NBLK];
-#pragma unroll
-        for (int nb = 0; nb < NBLK; ++nb) {
-            acc[nb] = v4f{0.f, 0.f, 0.f, 0.f};
-            gs[nb] = 0.f;
-            cn[nb] = 0.f;
-        }
-        float s1 = 0.f, s2 = 0.f;
-
-        // item l of this thread: float4 c4 of tile row `row`; rows beyond T / E are clamped (their
-        // scores are never used), items beyond the tile repeat its last one
-        const float* rptr[NL];
-        int lds_off[NL], kcol[NL];
-#pragma unroll
-        for (int l = 0; l < NL; ++l) {
-            const int idx = min(tid + l * kThreads, ROWS * KC4 - 1);
-            const int row = idx / KC4, c4 = idx % KC4;
-            rptr[l] = row < kTokens ? X + (size_t)min(t0 + row, T - 1) * d
-                      : row < kTokens + EP ? (PRE ? Cf : C) + (size_t)min(e0 + row - kTokens, E - 1) * d
-                                           : gamma;
-            lds_off[l] = row * LD + 4 * c4;
-            kcol[l] = 4 * c4;
-        }
-        // Two register sets: the loads of step s + 2 are issued before the arithmetic of step s and
-        // written to LDS one step later, so about two steps' worth of bytes (2 x 49 KB for 32
-        // experts) is in flight per CU - the arithmetic of one step is far shorter than a memory
-        // round trip and would not cover it.
-        v4f rg[2][NL];
-        auto load_step = [&](auto setc, int k0) {
-            constexpr int P = decltype(setc)::value;
-#pragma unroll
-            for (int l = 0; l < NL; ++l) rg[P][l] = load4<VEC>(rptr[l], k0 + kcol[l], d);
-        };
-        auto store_step = [&](auto setc, int buf, int k0) {
-            constexpr int P = decltype(setc)::value;
-            const v4f zero = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int l = 0; l < NL; ++l)  // k beyond the row was read from a clamped address: store zeros
-                *reinterpret_cast<v4f*>(s_tile + buf * (ROWS * LD) + lds_off[l]) = (k0 + kcol[l] < d) ? rg[P][l] : zero;
-        };
-        auto compute_step = [&](int buf) {
-            const float* tile = s_tile + buf * (ROWS * LD) + wave * (KC / kWaves) + 4 * kq;
-#pragma unroll
-            for (int g = 0; g < KC / kWaves / 16; ++g) {
-                const v4f xv = *reinterpret_cast<const v4f*>(tile + i * LD + 16 * g);
-                v4f gv = {1.f, 1.f, 1.f, 1.f};
-                if (GROW) gv = *reinterpret_cast<const v4f*>(tile + (kTokens + EP) * LD + 16 * g);
-                s1 += (xv.x + xv.y) + (xv.z + xv.w);
-                s2 += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
-#pragma unroll
-                for (int nb = 0; nb < NBLK; ++nb) {
-                    v4f cv = *reinterpret_cast<const v4f*>(tile + (kTokens + 16 * nb + i) * LD + 16 * g);
-                    if (!PRE) {
-                        cv *= gv;
-                        gs[nb] += (cv.x + cv.y) + (cv.z + cv.w);
-                        cn[nb] += (cv.x * cv.x + cv.y * cv.y) + (cv.z * cv.z + cv.w * cv.w);
-                    }
-                    // The k order inside a 16-float group is permuted identically for A and B, which
-                    // a dot product does not see: step j multiplies element j of every lane's float4.
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.x, cv.x, acc[nb], 0, 0, 0);
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.y, cv.y, acc[nb], 0, 0, 0);
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.z, cv.z, acc[nb], 0, 0, 0);
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv.w, cv.w, acc[nb], 0, 0, 0);
-                }
-            }
-        };
-        // step s computes from buffer s & 1; set P holds step s + 1, the other set receives step s + 2
-        auto step = [&](auto setc, int s) {
-            constexpr int P = decltype(setc)::value;
-            load_step(std::integral_constant<int, 1 - P>{}, min(s + 2, nsteps - 1) * KC);
-            compute_step(s & 1);
-            store_step(setc, (s + 1) & 1, (s + 1) * KC);
-            __syncthreads();
-        };
-        const std::integral_constant<int, 0> set0{};
-        const std::integral_constant<int, 1> set1{};
-        __syncthreads();  // the previous pass is done with the tile
-        load_step(set1, 0);
-        store_step(set1, 0, 0);
-        load_step(set0, min(1, nsteps - 1) * KC);
-        __syncthreads();
-        for (int s = 0; s < nsteps; s += 2) {
-            step(set0, s);
-            if (s + 1 < nsteps) step(set1, s + 1);
-        }
-
-        // lanes i, i+16, i+32, i+48 hold the four float4 slots of one row
-        s1 += __shfl_xor(s1, 16);
-        s1 += __shfl_xor(s1, 32);
-        s2 += __shfl_xor(s2, 16);
-        s2 += __shfl_xor(s2, 32);
-        if (kq == 0) {
-            s_s1[wave][i] = s1;
-            s_s2[wave][i] = s2;
-        }
-#pragma unroll
-        for (int nb = 0; nb < NBLK; ++nb) {
-            float g = gs[nb], n2 = cn[nb];
-            g += __shfl_xor(g, 16);
-            g += __shfl_xor(g, 32);
-            n2 += __shfl_xor(n2, 16);
-            n2 += __shfl_xor(n2, 32);
-            if (kq == 0) {
-                s_g1[wave][16 * nb + i] = g;
-                s_g2[wave][16 * nb + i] = n2;
-            }
-            // D layout of 16x16x4: lane holds column (lane & 15), rows 4*(lane >> 4) + r
-#pragma unroll
-            for (int r = 0; r < 4; ++r) s_part[wave][4 * kq + r][16 * nb + i] = acc[nb][r];
-        }
-        __syncthreads();
-
-        if (tid < kTokens) {
-            float a1 = 0.f, a2 = 0.f;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) a1 += s_s1[w][tid], a2 += s_s2[w][tid];
+    // Scores of the pass over experts e0 .. e0+EP from what is in LDS: raw dot products in s_score, raw
+    // row sums in s_a1 / s_a2, and (without PRE) the centroid sums in s_G and sums of squares in s_cn.
+    auto finish_pass = [&](int e0) {
+        if (tid < TM) {
+            const float a1 = s_a1[tid], a2 = s_a2[tid];
             float mu = 0.f, rstd = 1.f;
             if (norm_kind == NORM_RMS) {
                 rstd = 1.0f / sqrtf(a2 / (float)d + kNormEps);
@@ -250,41 +196,34 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
             const int e = tid - 64;
             if (PRE) {
                 const int ee = min(e0 + e, E - 1);
-                s_G[e] = cstats[ee];
-                s_cn[e] = cstats[E + ee];
+                s_G[e] = arg.cstats[ee];
+                s_cn[e] = arg.cstats[E + ee];
             } else {
-                float g1 = 0.f, g2 = 0.f;
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) g1 += s_g1[w][e], g2 += s_g2[w][e];
-                s_G[e] = g1;
-                s_cn[e] = sqrtf(g2);
+                s_cn[e] = sqrtf(s_cn[e]);
             }
         }
         __syncthreads();
-
-        for (int idx = tid; idx < kTokens * EP; idx += kThreads) {
+        for (int idx = tid; idx < TM * EP; idx += kThreads) {
             const int tok = idx / EP, e = idx - tok * EP;
-            float dot = 0.f;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) dot += s_part[w][tok][e];
-            float sc = s_rstd[tok] * (dot - s_mu[tok] * s_G[e]);
+            float sc = s_rstd[tok] * (s_score[tok][e] - s_mu[tok] * s_G[e]);
             if (bias != nullptr && e0 + e < E) sc += bias[e0 + e];
             s_score[tok][e] = sc;
         }
         __syncthreads();
 
-        // each wave reduces kTokens / kWaves tokens
         const int nvalid = min(E - e0, EP);
         float cmax = 0.f;
         for (int e = lane; e < nvalid; e += 64) cmax = fmaxf(cmax, s_cn[e]);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) cmax = fmaxf(cmax, __shfl_xor(cmax, off));
         if (tid == 0) s_cnmax = fmaxf(s_cnmax, cmax);
-        for (int q = 0; q < kTokens / kWaves; ++q) {
-            const int tok = (kTokens / kWaves) * wave + q;
+        // 16 lanes reduce one token; a wave takes four tokens at a time
+#pragma unroll 1
+        for (int q = 0; q < MB; ++q) {
+            const int tok = (TM / kWaves) * wave + 4 * q + kq;
             float v = -FLT_MAX;
             int vi = -1;
-            for (int e = lane; e < nvalid; e += 64) {
+            for (int e = i; e < nvalid; e += 16) {
                 const float s = s_score[tok][e];
                 if (s > v) {
                     v = s;
@@ -292,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
                 }
             }
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
+            for (int off = 8; off > 0; off >>= 1) {
                 const float ov = __shfl_xor(v, off);
                 const int oi = __shfl_xor(vi, off);
                 if (ov > v || (ov == v && (unsigned)oi < (unsigned)vi)) {
@@ -301,13 +240,13 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
                 }
             }
             float v2 = -FLT_MAX;
-            for (int e = lane; e < nvalid; e += 64) {
+            for (int e = i; e < nvalid; e += 16) {
                 const float s = s_score[tok][e];
                 if (e0 + e != vi && s > v2) v2 = s;
             }
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v2 = fmaxf(v2, __shfl_xor(v2, off));
-            if (lane == 0) {
+            for (int off = 8; off > 0; off >>= 1) v2 = fmaxf(v2, __shfl_xor(v2, off));
+            if (i == 0) {
                 const float B = s_best[tok];
                 if (v > B) {
                     s_second[tok] = fmaxf(B, v2);
@@ -319,13 +258,246 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
             }
         }
         __syncthreads();
+    };
+
+    for (int e0 = 0; mode != GATE_COMBINE && e0 < E; e0 += EP) {
+        v4f acc[2][NBLK];  // two sets, for even and odd 16-float groups: twice as many independent chains
+        float gs[NBLK], cn[NBLK], s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < NBLK; ++nb) {
+            acc[0][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+            acc[1][nb] = v4f{0.f, 0.f, 0.f, 0.f};
+            gs[nb] = 0.f;
+            cn[nb] = 0.f;
+        }
+
+        // item l of this thread: float4 c4 of tile row `row`; rows beyond T / E are clamped (their
+        // scores are never used), items beyond the tile repeat its last one
+        const float* rptr[NL];
+        int lds_off[NL], kcol[NL];
+#pragma unroll
+        for (int l = 0; l < NL; ++l) {
+            const int idx = min(tid + l * kThreads, ROWS * KC4 - 1);
+            const int row = idx / KC4, c4 = idx % KC4;
+            rptr[l] = row < TM ? X + (size_t)min(t0 + row, T - 1) * d
+                      : row < TM + EP ? (PRE ? arg.Cf : C) + (size_t)min(e0 + row - TM, E - 1) * d
+                                      : gamma;
+            lds_off[l] = row * LD + 4 * c4;
+            kcol[l] = 4 * c4;
+        }
+        // Two register sets: the loads of step s + 2 are issued before the arithmetic of step s and
+        // written to LDS one step later, so about two steps' worth of bytes is in flight per CU - the
+        // arithmetic of one step is shorter than a memory round trip and would not cover it.
+        v4f rg[2][NL];
+        auto load_step = [&](auto setc, int sl) {
+            constexpr int P = decltype(setc)::value;
+            const int k0 = k_lo + min(sl, nst - 1) * KC;
+#pragma unroll
+            for (int l = 0; l < NL; ++l) rg[P][l] = load4<VEC>(rptr[l], k0 + kcol[l], d);
+        };
+        auto store_step = [&](auto setc, int buf, int sl) {
+            constexpr int P = decltype(setc)::value;
+            const int k0 = k_lo + sl * KC;
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int l = 0; l < NL; ++l)  // k beyond the slice was read from a clamped address: store zeros
+                *reinterpret_cast<v4f*>(s_tile + buf * (ROWS * LD) + lds_off[l]) = (k0 + kcol[l] < k_hi) ? rg[P][l] : zero;
+        };
+        auto compute_step = [&](int buf) {
+            // SPLITK: this wave's quarter of the chunk, token rows 0..15; otherwise the whole chunk and
+            // token rows 16*wave .. 16*wave+15
+            constexpr int NG = (SPLITK ? KC / kWaves : KC) / 16;
+            const float* tile = s_tile + buf * (ROWS * LD) + (SPLITK ? wave * (KC / kWaves) : 0) + 4 * kq;
+            const float* xrow = tile + ((SPLITK ? 0 : 16 * wave) + i) * LD;
+#pragma unroll
+            for (int gq = 0; gq < NG; ++gq) {
+                const v4f xv = *reinterpret_cast<const v4f*>(xrow + 16 * gq);
+                v4f gv = {1.f, 1.f, 1.f, 1.f};
+                if (GROW) gv = *reinterpret_cast<const v4f*>(tile + (TM + EP) * LD + 16 * gq);
+                s1 += (xv.x + xv.y) + (xv.z + xv.w);
+                s2 += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
+                v4f cv[NBLK];
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    cv[nb] = *reinterpret_cast<const v4f*>(tile + (TM + 16 * nb + i) * LD + 16 * gq);
+                    if (!PRE) {
+                        cv[nb] *= gv;
+                        gs[nb] += (cv[nb].x + cv[nb].y) + (cv[nb].z + cv[nb].w);
+                        cn[nb] += (cv[nb].x * cv[nb].x + cv[nb].y * cv[nb].y) + (cv[nb].z * cv[nb].z + cv[nb].w * cv[nb].w);
+                    }
+                }
+                // The k order inside a 16-float group is permuted identically for A and B, which a dot
+                // product does not see: step c multiplies element c of every lane's float4.  Consecutive
+                // instructions go to different accumulators so that none waits for its predecessor.
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb)
+                        acc[gq & 1][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[c], cv[nb][c], acc[gq & 1][nb], 0, 0, 0);
+            }
+        };
+        // step sl computes from buffer sl & 1; set P holds step sl + 1, the other set receives step sl + 2
+        auto step = [&](auto setc, int sl) {
+            constexpr int P = decltype(setc)::value;
+            load_step(std::integral_constant<int, 1 - P>{}, sl + 2);
+            __builtin_amdgcn_sched_barrier(0);  // the loads go out before the arithmetic, not next to their use
+            compute_step(sl & 1);
+            store_step(setc, (sl + 1) & 1, sl + 1);
+            __syncthreads();
+        };
+        const std::integral_constant<int, 0> set0{};
+        const std::integral_constant<int, 1> set1{};
+        __syncthreads();  // the previous pass is done with the tile
+        load_step(set1, 0);
+        store_step(set1, 0, 0);
+        load_step(set0, 1);
+        __syncthreads();
+        // Steps go in pairs without a branch between them: a conditional second step is a block of its
+        // own, and the compiler then moves the first step's loads down into it, next to the LDS stores
+        // that use them, which exposes a full memory round trip per pair.  With an odd number of
+        // chunks the last step works on a tile of zeros (its predecessor stored k >= k_hi as zeros).
+        for (int sl = 0; sl < nst; sl += 2) {
+            step(set0, sl);
+            step(set1, sl + 1);
+        }
+
+        // lanes i, i+16, i+32, i+48 hold the four float4 slots of one row
+        s1 += __shfl_xor(s1, 16);
+        s1 += __shfl_xor(s1, 32);
+        s2 += __shfl_xor(s2, 16);
+        s2 += __shfl_xor(s2, 32);
+        if (kq == 0) {
+            s_s1[wave][i] = s1;
+            s_s2[wave][i] = s2;
+        }
+#pragma unroll
+        for (int nb = 0; nb < NBLK; ++nb) {
+            float gsum = gs[nb], n2 = cn[nb];
+            gsum += __shfl_xor(gsum, 16);
+            gsum += __shfl_xor(gsum, 32);
+            n2 += __shfl_xor(n2, 16);
+            n2 += __shfl_xor(n2, 32);
+            if (kq == 0) {
+                s_g1[wave][16 * nb + i] = gsum;
+                s_g2[wave][16 * nb + i] = n2;
+            }
+            // D layout of 16x16x4: lane holds column (lane & 15), rows 4*(lane >> 4) + r
+            const v4f sum = acc[0][nb] + acc[1][nb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (SPLITK) s_part[wave][4 * kq + r][16 * nb + i] = sum[r];
+                else s_score[16 * wave + 4 * kq + r][16 * nb + i] = sum[r];
+            }
+        }
+        __syncthreads();
+        if (SPLITK) {  // the four waves hold partial sums over K of the same 16 tokens
+            for (int idx = tid; idx < 16 * EP; idx += kThreads) {
+                const int tok = idx / EP, e = idx - tok * EP;
+                float dot = 0.f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) dot += s_part[SPLITK ? w : 0][SPLITK ? tok : 0][SPLITK ? e : 0];
+                s_score[tok][e] = dot;
+            }
+        }
+        if (tid < TM) {
+            float a1 = 0.f, a2 = 0.f;
+            if (SPLITK) {
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) a1 += s_s1[w][tid], a2 += s_s2[w][tid];
+            } else {  // wave tid / 16 owns this token
+                a1 = s_s1[tid >> 4][tid & 15], a2 = s_s2[tid >> 4][tid & 15];
+            }
+            s_a1[tid] = a1;
+            s_a2[tid] = a2;
+        } else if (!PRE && tid >= 64 && tid < 64 + EP) {
+            const int e = tid - 64;
+            float g1 = 0.f, g2 = 0.f;
+            if (SPLITK) {
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) g1 += s_g1[w][e], g2 += s_g2[w][e];
+            } else {  // every wave saw all of K
+                g1 = s_g1[0][e], g2 = s_g2[0][e];
+            }
+            s_G[e] = g1;
+            s_cn[e] = g2;
+        }
+        __syncthreads();
+
+        if (mode == GATE_WHOLE) {
+            finish_pass(e0);
+        } else {
+            // this slice's share of the pass goes to scratch memory
+            float* part = arg.partials + (size_t)j * T * W;
+            for (int idx = tid; idx < TM * EP; idx += kThreads) {
+                const int tok = idx / EP, e = idx - tok * EP;
+                if (t0 + tok < T && e0 + e < E) part[(size_t)(t0 + tok) * W + e0 + e] = s_score[tok][e];
+            }
+            if (e0 == 0 && tid < TM && t0 + tid < T) {
+                part[(size_t)(t0 + tid) * W + E] = s_a1[tid];
+                part[(size_t)(t0 + tid) * W + E + 1] = s_a2[tid];
+            }
+            if (!PRE && tid >= 64 && tid < 64 + EP && e0 + tid - 64 < E) {
+                float* gp = arg.gpart + ((size_t)g * S + j) * 2 * E;
+                gp[e0 + tid - 64] = s_G[tid - 64];
+                gp[E + e0 + tid - 64] = s_cn[tid - 64];
+            }
+            if (e0 + EP < E) __syncthreads();  // the next pass overwrites what is being read here
+        }
+    }
+
+    if (mode == GATE_SLICES) return;
+    if (mode == GATE_COMBINE) {
+        for (int e0 = 0; e0 < E; e0 += EP) {
+            for (int idx = tid; idx < TM * EP; idx += kThreads) {
+                const int tok = idx / EP, e = idx - tok * EP;
+                float sum = 0.f;
+                if (t0 + tok < T && e0 + e < E) {
+                    // all slices' loads go out together (a loop over a run-time count waits for each
+                    // in turn); the sum is taken in slice order
+                    const float* src = arg.partials + (size_t)(t0 + tok) * W + e0 + e;
+                    float v[kMaxSlices];
+#pragma unroll
+                    for (int jj = 0; jj < kMaxSlices; ++jj) v[jj] = src[(size_t)min(jj, S - 1) * T * W];
+#pragma unroll
+                    for (int jj = 0; jj < kMaxSlices; ++jj) sum += jj < S ? v[jj] : 0.f;
+                }
+                s_score[tok][e] = sum;
+            }
+            if (tid < TM) {
+                float a1 = 0.f, a2 = 0.f;
+                if (t0 + tid < T) {
+                    const float* src = arg.partials + (size_t)(t0 + tid) * W + E;
+                    float v1[kMaxSlices], v2[kMaxSlices];
+#pragma unroll
+                    for (int jj = 0; jj < kMaxSlices; ++jj) {
+                        v1[jj] = src[(size_t)min(jj, S - 1) * T * W];
+                        v2[jj] = src[(size_t)min(jj, S - 1) * T * W + 1];
+                    }
+#pragma unroll
+                    for (int jj = 0; jj < kMaxSlices; ++jj) a1 += jj < S ? v1[jj] : 0.f, a2 += jj < S ? v2[jj] : 0.f;
+                }
+                s_a1[tid] = a1;
+                s_a2[tid] = a2;
+            } else if (!PRE && tid >= 64 && tid < 64 + EP) {
+                const int e = tid - 64;
+                float g1 = 0.f, g2 = 0.f;
+                if (e0 + e < E) {
+                    const float* src = arg.gpart + (size_t)g * S * 2 * E + e0 + e;
+                    for (int jj = 0; jj < S; ++jj) g1 += src[(size_t)jj * 2 * E], g2 += src[(size_t)jj * 2 * E + E];
+                }
+                s_G[e] = g1;
+                s_cn[e] = g2;
+            }
+            __syncthreads();
+            finish_pass(e0);
+        }
     }
 
     // ---- decide, per token, whether FP32 ordered the top two safely
-    if (tid < kTokens) {
+    if (tid < TM) {
         const int t = t0 + tid;
         if (t < T) {
-            const float B = s_best[tid], S = s_second[tid];
+            const float B = s_best[tid], S2 = s_second[tid];
             const int I = s_besti[tid];
             if (I < 0) {  // no orderable score: the reference asserts (plugin/cuda/moe.cu:70)
                 sel[t] = 0;
@@ -336,7 +508,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
                 coeff[t] = B;
                 const float bound = 8.f * FLT_EPSILON * s_rstd[tid] * s_xnorm[tid] * s_cnmax;
                 s_thr[tid] = fmaxf(bound, 4e-6f * fabsf(B));
-                if (E > 1 && (B - S) < s_thr[tid]) s_rescue[tid] = 1;
+                if (E > 1 && (B - S2) < s_thr[tid]) s_rescue[tid] = 1;
             }
         }
     }
@@ -344,7 +516,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
 
     // ---- float64 re-scoring of the flagged tokens by the whole workgroup: the waves share the
     // row statistics, then each wave takes every kWaves-th expert and the scores meet in LDS
-    for (int tok = 0; tok < kTokens; ++tok) {
+    for (int tok = 0; tok < TM; ++tok) {
         if (!s_rescue[tok]) continue;  // uniform: read from LDS after the barrier
         // Quick path (one pass over experts, at most kMaxCand experts within the bound of the best):
         // only those candidates can win, so one sweep over d computes, in float64, the row statistics
@@ -553,53 +725,124 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(int T, int d, int E
     }
 }
 
+// How a call is split into workgroups.
+struct GatePlan {
+    int mb;         // 16-token blocks per workgroup: 1 or 4
+    int groups;     // token groups
+    int slices;     // workgroups per token group
+    int steps_per;  // K chunks per slice
+};
+
+constexpr int nblk_for(int E) { return E <= 16 ? 1 : (E <= 32 ? 2 : (E <= 64 ? 4 : 8)); }
+
+GatePlan gate_plan(int T, int d, int E, bool vec, size_t scratch_floats) {
+    const int nblk = nblk_for(E);
+    const int W = E + 2;
+    auto slices_for = [&](int mb, GatePlan* p) {
+        const int kc = gate_kc(nblk, mb);
+        const int nsteps = (d + kc - 1) / kc;
+        const int groups = (T + 16 * mb - 1) / (16 * mb);
+        int want = (kTargetGroups + groups - 1) / groups;
+        want = std::min(want, std::min(kMaxSlices, nsteps));
+        want = std::min(want, std::max(1, d / (2 * W)));  // partial sums stay a fraction of the input's bytes
+        const int per = (nsteps + want - 1) / want;
+        p->mb = mb, p->groups = groups, p->steps_per = per, p->slices = (nsteps + per - 1) / per;
+        if (p->slices > 1 && (size_t)p->slices * T * W + (size_t)groups * p->slices * 2 * E > scratch_floats) {
+            p->slices = 1;
+            p->steps_per = nsteps;
+        }
+    };
+    GatePlan wide{}, narrow{};
+    slices_for(1, &narrow);
+    if (!vec || T < 64 * kTargetGroups) return narrow;
+    // 64-token workgroups move a quarter of the centroid bytes per token; take them when they give
+    // every compute unit a workgroup without slicing (measured at 4096 tokens x 4096 x 32 experts:
+    // 64 tokens x 4 slices 46 us, 16 tokens unsliced 32 us)
+    slices_for(4, &wide);
+    wide.slices = 1;
+    wide.steps_per = (d + gate_kc(nblk, 4) - 1) / gate_kc(nblk, 4);
+    return wide;
+}
+
 template <int NBLK>
-hipError_t launch_nblk(int T, int d, int E, const float* x, const float* c, const float* gamma, const float* cf,
-                       const float* cstats, int norm_kind, const float* bias, int* sel, float* coeff, int* stats,
-                       hipStream_t stream) {
-    const dim3 grid((T + kTokens - 1) / kTokens), block(kThreads);
-    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(c) |
-                           reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(cf)) & 15) == 0;
-    const bool pre = cf != nullptr && cstats != nullptr;
-    const bool vec = d % 4 == 0 && aligned;
-    const bool use_gamma = norm_kind != NORM_NONE && gamma != nullptr;
-    constexpr int KC = NBLK <= 2 ? 256 : (NBLK == 4 ? 128 : 64);
+hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const GatePlan& plan, hipStream_t stream) {
+    a.slices = plan.slices, a.steps_per = plan.steps_per;
+    const dim3 block(kThreads);
     hipError_t err = hipSuccess;
-#define INFMOE_GATE(V, G, P)                                                                                       \
-    do {                                                                                                           \
-        const size_t lds = 2 * (size_t)(kTokens + 16 * NBLK + ((G) && !(P) ? 1 : 0)) * (KC + 4) * sizeof(float);   \
-        err = allow_lds_once<gate_top1_kernel<NBLK, V, G, P>>(lds);                                                \
-        if (err != hipSuccess) return err;                                                                         \
-        gate_top1_kernel<NBLK, V, G, P><<<grid, block, lds, stream>>>(T, d, E, x, c, gamma, cf, cstats, norm_kind, \
-                                                                      bias, sel, coeff, stats);                    \
+#define INFMOE_GATE(M, V, G, P)                                                                                   \
+    do {                                                                                                          \
+        constexpr int KC = gate_kc(NBLK, M);                                                                      \
+        const size_t lds = 2 * (size_t)(16 * (M) + 16 * NBLK + ((G) && !(P) ? 1 : 0)) * (KC + 4) * sizeof(float); \
+        err = allow_lds_once<gate_top1_kernel<NBLK, M, V, G, P>>(lds);                                            \
+        if (err != hipSuccess) return err;                                                                        \
+        if (plan.slices == 1) {                                                                                   \
+            a.mode = GATE_WHOLE;                                                                                  \
+            gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups), block, lds, stream>>>(a);                     \
+        } else {                                                                                                  \
+            a.mode = GATE_SLICES;                                                                                 \
+            gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups * plan.slices), block, lds, stream>>>(a);       \
+            a.mode = GATE_COMBINE; /* does not touch the staging tile */                                          \
+            gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups), block, 0, stream>>>(a);                       \
+        }                                                                                                         \
+    } while (0)
+#define INFMOE_GATE_M(V, G, P)                     \
+    do {                                           \
+        if (plan.mb == 4) INFMOE_GATE(4, V, G, P); \
+        else INFMOE_GATE(1, V, G, P);              \
     } while (0)
     if (vec && pre) {  // the layer's path: 16-byte rows and precomputed centroid data
-        if (use_gamma) INFMOE_GATE(true, true, true);
-        else INFMOE_GATE(true, false, true);
+        if (use_gamma) INFMOE_GATE_M(true, true, true);
+        else INFMOE_GATE_M(true, false, true);
     } else if (vec) {
-        if (use_gamma) INFMOE_GATE(true, true, false);
-        else INFMOE_GATE(true, false, false);
-    } else {
-        if (use_gamma) INFMOE_GATE(false, true, false);
-        else INFMOE_GATE(false, false, false);
+        if (use_gamma) INFMOE_GATE_M(true, true, false);
+        else INFMOE_GATE_M(true, false, false);
+    } else {  // rows that are not 16-byte aligned: 16-token workgroups only
+        if (use_gamma) INFMOE_GATE(1, false, true, false);
+        else INFMOE_GATE(1, false, false, false);
     }
+#undef INFMOE_GATE_M
 #undef INFMOE_GATE
     return hipGetLastError();
 }
 
 }  // namespace
 
+size_t gate_scratch_floats(int T, int d, int E) {
+    // Enough for every call of up to T tokens.  Only 16-token workgroups are sliced, and only while
+    // there are fewer than kTargetGroups token groups: slices * tokens <= (kTargetGroups / groups + 1)
+    // * groups * 16 <= 16 * kTargetGroups + tokens + 16, and groups * slices <= 2 * kTargetGroups.
+    const int kc = gate_kc(nblk_for(E), 1);
+    const size_t W = (size_t)E + 2;
+    const size_t max_slices = std::min<size_t>(std::min(kMaxSlices, (d + kc - 1) / kc), std::max<size_t>(1, (size_t)d / (2 * W)));
+    if (max_slices <= 1 || T <= 0) return 0;
+    const size_t tokens = std::min(T, 16 * kTargetGroups);
+    const size_t rows = std::min(max_slices * tokens, (size_t)16 * kTargetGroups + tokens + 16);
+    return rows * W + (size_t)2 * kTargetGroups * 2 * (size_t)E;
+}
+
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
-                            hipStream_t stream, const float* folded_centroids, const float* centroid_stats) {
+                            hipStream_t stream, const float* folded_centroids, const float* centroid_stats,
+                            float* scratch, size_t scratch_floats) {
     if (T <= 0) return hipSuccess;
-#define INFMOE_NBLK(n) \
-    return launch_nblk<n>(T, d, E, x, centroids, gamma, folded_centroids, centroid_stats, norm_kind, score_bias, sel, coeff, stats, stream)
-    if (E <= 16) INFMOE_NBLK(1);
-    if (E <= 32) INFMOE_NBLK(2);
-    if (E <= 64) INFMOE_NBLK(4);
-    INFMOE_NBLK(8);
-#undef INFMOE_NBLK
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(centroids) |
+                           reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(folded_centroids)) & 15) == 0;
+    const bool pre = folded_centroids != nullptr && centroid_stats != nullptr;
+    const bool vec = d % 4 == 0 && aligned;
+    const bool use_gamma = norm_kind != NORM_NONE && gamma != nullptr;
+    const GatePlan plan = gate_plan(T, d, E, vec, scratch != nullptr ? scratch_floats : 0);
+    GateArgs a{};
+    a.T = T, a.d = d, a.E = E;
+    a.X = x, a.C = centroids, a.gamma = gamma, a.Cf = folded_centroids, a.cstats = centroid_stats;
+    a.norm_kind = norm_kind, a.bias = score_bias, a.sel = sel, a.coeff = coeff, a.stats = stats;
+    a.partials = scratch;
+    a.gpart = scratch ? scratch + (size_t)plan.slices * T * (E + 2) : nullptr;
+    switch (nblk_for(E)) {
+        case 1: return launch_nblk<1>(a, vec, pre, use_gamma, plan, stream);
+        case 2: return launch_nblk<2>(a, vec, pre, use_gamma, plan, stream);
+        case 4: return launch_nblk<4>(a, vec, pre, use_gamma, plan, stream);
+        default: return launch_nblk<8>(a, vec, pre, use_gamma, plan, stream);
+    }
 }
 
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats) {

@@ -21,10 +21,15 @@ constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/subla
 // Optional: folded_centroids [E][d] = centroids * gamma (device) and centroid_stats [2E] = per expert
 // the sum and the Euclidean norm of that product (device), both made by fold_centroids_host; with
 // them the kernel skips work that depends on the layer's parameters only.
+// Optional: scratch (gate_scratch_floats(T, d, E) floats, any contents): with it the embedding dimension
+// of a call with few tokens is split over several workgroups per token group, and a second launch adds
+// their partial scores and selects.
+size_t gate_scratch_floats(int T, int d, int E);
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids = nullptr,
-                            const float* centroid_stats = nullptr);
+                            const float* centroid_stats = nullptr, float* scratch = nullptr,
+                            size_t scratch_floats = 0);
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)

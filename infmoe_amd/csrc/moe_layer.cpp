@@ -125,6 +125,7 @@ struct MoELayer::Carve {
     RowTile* tiles = nullptr;
     int maxTiles = 0;
     void* countScratch = nullptr;
+    float* gateScratch = nullptr;  // partial scores of the gating kernel's slices
     float *coeff = nullptr, *routedCoeff = nullptr, *routed = nullptr, *post = nullptr;
     size_t total = 0;
 };
@@ -154,6 +155,7 @@ Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     c->tiles = reinterpret_cast<RowTile*>(take(sizeof(RowTile) * 2 * (size_t)c->maxTiles));
     c->sched = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kSchedInts));
     c->countScratch = take(expert_count_scratch_bytes(T, E));
+    c->gateScratch = reinterpret_cast<float*>(take(sizeof(float) * gate_scratch_floats(T, d, E)));
     c->coeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
     c->routedCoeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
     c->routed = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T * d));
@@ -282,7 +284,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     const bool ln = mParams.flags.layernormOnInputBeforeScore;
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
                                 mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream, mFoldedGpu,
-                                mFoldedGpu + (size_t)E * d));
+                                mFoldedGpu + (size_t)E * d, c.gateScratch, gate_scratch_floats(T, d, E)));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     const bool grouped = resident();

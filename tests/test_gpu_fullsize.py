@@ -27,9 +27,10 @@ def device_gate(lib, torch, x2d, cent, gamma, norm, bias):
     coeff = torch.empty(T, dtype=torch.float32, device="cuda")
     stats = torch.zeros(4, dtype=torch.int32, device="cuda")
     db = torch.from_numpy(bias).cuda() if bias is not None else None
+    ws = torch.empty(max(lib.infmoe_gate_top1_scratch_bytes(T, d, E), 16), dtype=torch.uint8, device="cuda")
     capi.check(lib.infmoe_gate_top1(T, d, E, x2d.data_ptr(), cent.data_ptr(), gamma.data_ptr() if norm != "none" else None,
                                     capi.NORM_KINDS[norm], db.data_ptr() if db is not None else None, sel.data_ptr(),
-                                    coeff.data_ptr(), stats.data_ptr(), stream_ptr(torch)))
+                                    coeff.data_ptr(), stats.data_ptr(), ws.data_ptr(), stream_ptr(torch)))
     torch.cuda.synchronize()
     return sel.cpu().numpy(), coeff.cpu().numpy(), stats.cpu().numpy()
 

@@ -12,7 +12,9 @@ FFN = capi.FFN_KINDS
 
 
 # ------------------------------------------------------------------ gating
-def run_gate(lib, torch, x, c, gamma, norm, bias=None):
+def run_gate(lib, torch, x, c, gamma, norm, bias=None, scratch=True):
+    """scratch=True hands over the optional scratch memory (filled with 0xFF bytes: any contents are
+    allowed), which lets the kernel split the embedding dimension; False runs the one-pass form."""
     T, d = x.shape
     E = c.shape[0]
     dx, dc = dev(torch, x), dev(torch, c)
@@ -21,9 +23,11 @@ def run_gate(lib, torch, x, c, gamma, norm, bias=None):
     sel = torch.full((T,), -7, dtype=torch.int32, device="cuda")
     coeff = torch.zeros(T, dtype=torch.float32, device="cuda")
     stats = torch.zeros(4, dtype=torch.int32, device="cuda")
+    ws = torch.full((max(lib.infmoe_gate_top1_scratch_bytes(T, d, E), 16),), 255, dtype=torch.uint8, device="cuda") if scratch else None
     capi.check(lib.infmoe_gate_top1(T, d, E, dx.data_ptr(), dc.data_ptr(), dg.data_ptr() if dg is not None else None,
                                     NORM[norm], db.data_ptr() if db is not None else None, sel.data_ptr(),
-                                    coeff.data_ptr(), stats.data_ptr(), stream_ptr(torch)))
+                                    coeff.data_ptr(), stats.data_ptr(), ws.data_ptr() if scratch else None,
+                                    stream_ptr(torch)))
     torch.cuda.synchronize()
     return sel.cpu().numpy(), coeff.cpu().numpy(), stats.cpu().numpy()
 
@@ -37,13 +41,18 @@ def run_gate(lib, torch, x, c, gamma, norm, bias=None):
     (300, 2048, 64, "none", True),   # base_layer shape with score bias
     (50, 512, 200, "centered", True),  # more than 128 experts: several passes
     (64, 4096, 32, "centered", False),
+    (2048, 2048, 16, "centered", False),  # 2 slices of the embedding dimension
+    (16389, 256, 8, "rms", True),         # 64-token workgroups, ragged last group
+    (40, 4096, 200, "rms", False),        # several passes over experts and several slices
+    (1024, 1024, 32, "rms", False),       # 16-token workgroups, 4 slices
 ])
-def test_gate_top1_matches_oracle(lib, torch_cuda, T, d, E, norm, use_bias):
+@pytest.mark.parametrize("scratch", [True, False])
+def test_gate_top1_matches_oracle(lib, torch_cuda, T, d, E, norm, use_bias, scratch):
     torch = torch_cuda
     x, c, g = O.draw_inputs(11, T, d, E)
     x = x + (0.3 if norm == "centered" else 0.0)  # a mean for the centred norm to remove
     bias = (0.2 * np.random.default_rng(5).standard_normal(E)).astype(np.float32) if use_bias else None
-    sel, coeff, stats = run_gate(lib, torch, x, c, g if norm != "none" else None, norm, bias)
+    sel, coeff, stats = run_gate(lib, torch, x, c, g if norm != "none" else None, norm, bias, scratch=scratch)
     xa = O.layernorm(x, g, norm) if norm != "none" else x.astype(np.float64)
     aff = O.score(xa, c, bias)
     exempt = check_assignment(sel, aff)
@@ -53,10 +62,11 @@ def test_gate_top1_matches_oracle(lib, torch_cuda, T, d, E, norm, use_bias):
     assert_close(coeff, want, what="coeff")
 
 
-def test_gate_top1_exact_ties_pick_lowest_index(lib, torch_cuda):
+@pytest.mark.parametrize("d", [32, 1024])  # one chunk; several slices
+def test_gate_top1_exact_ties_pick_lowest_index(lib, torch_cuda, d):
     torch = torch_cuda
     rng = np.random.default_rng(3)
-    T, d, E = 64, 32, 24
+    T, E = 64, 24
     x = rng.integers(-2, 3, size=(T, d)).astype(np.float32)  # small integers: scores are exact
     c = rng.integers(-1, 2, size=(E, d)).astype(np.float32)
     c[7] = c[3]
@@ -69,9 +79,10 @@ def test_gate_top1_exact_ties_pick_lowest_index(lib, torch_cuda):
     assert stats[0] == int((O.top2_relative_gap(aff) < 1e-6).sum())
 
 
-def test_gate_top1_counts_nan_rows(lib, torch_cuda):
+@pytest.mark.parametrize("d", [64, 2048])  # one chunk; several slices
+def test_gate_top1_counts_nan_rows(lib, torch_cuda, d):
     torch = torch_cuda
-    x, c, g = O.draw_inputs(2, 40, 64, 8)
+    x, c, g = O.draw_inputs(2, 40, d, 8)
     x[5, 3] = np.nan
     x[33, :] = np.nan
     sel, coeff, stats = run_gate(lib, torch, x, c, g, "rms")
