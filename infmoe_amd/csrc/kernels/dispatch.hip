@@ -16,6 +16,7 @@
 
 #include <initializer_list>
 
+#include "device_math.h"
 #include "kernels.h"
 
 namespace infmoe {
@@ -278,8 +279,12 @@ __global__ __launch_bounds__(kThreads) void mix_gather_kernel(int T, int d, cons
     const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (r >= T) return;
     // plugin/cuda/common.cuh:24-27 and plugin/cuda/moe.cu:120-126
-    const float a = 1.0f / (1.0f + expf(-routed_coeff[r]));
+    const float a = sigmoid_f(routed_coeff[r]);
     const float b = 1.0f - a;
+    auto mix4 = [&](const v4f& pv, const v4f& qv) {
+        return v4f{mix_value(a, b, pv.x, qv.x), mix_value(a, b, pv.y, qv.y), mix_value(a, b, pv.z, qv.z),
+                   mix_value(a, b, pv.w, qv.w)};
+    };
     const float* p = post + (size_t)r * d;
     const float* q = routed + (size_t)r * d;
     float* o = out + (size_t)pos[r] * d;
@@ -291,12 +296,12 @@ __global__ __launch_bounds__(kThreads) void mix_gather_kernel(int T, int d, cons
         int k = lane;
         for (; k + 64 < n4; k += 128) {
             const v4f p0 = p4[k], p1 = p4[k + 64], q0 = q4[k], q1 = q4[k + 64];
-            o4[k] = a * p0 + b * q0;
-            o4[k + 64] = a * p1 + b * q1;
+            o4[k] = mix4(p0, q0);
+            o4[k + 64] = mix4(p1, q1);
         }
-        for (; k < n4; k += 64) o4[k] = a * p4[k] + b * q4[k];
+        for (; k < n4; k += 64) o4[k] = mix4(p4[k], q4[k]);
     } else {
-        for (int k = lane; k < d; k += 64) o[k] = a * p[k] + b * q[k];
+        for (int k = lane; k < d; k += 64) o[k] = mix_value(a, b, p[k], q[k]);
     }
 }
 

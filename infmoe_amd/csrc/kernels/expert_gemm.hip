@@ -334,17 +334,20 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProbl
 }
 
 // Shapes the matrix-core kernel does not take (K not a multiple of 32, or operands that are not
-// 16-byte aligned): one thread per output element.  Only tiny debug shapes come here.
-__global__ void expert_gemm_generic_kernel(GemmProblem p, int rows) {
+// 16-byte aligned): one thread per output element.  Only small or odd shapes come here.
+// row_expert == nullptr: one expert; else row r uses the weights of expert row_expert[r].
+__global__ void expert_gemm_generic_kernel(GemmProblem p, int rows, size_t weight_stride,
+                                           const int* __restrict__ row_expert) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)rows * p.N) return;
     const int row = idx / p.N, col = idx % p.N;
+    const size_t w0 = row_expert ? (size_t)row_expert[row] * weight_stride : 0;
     const float* a = p.A + (size_t)row * p.K;
-    const float* b0 = p.B + (size_t)col * p.K;
+    const float* b0 = p.B + w0 + (size_t)col * p.K;
     float s0 = 0.f, s1 = 0.f;
     for (int k = 0; k < p.K; ++k) s0 += a[k] * b0[k];
     if (p.epilogue == EPI_GATED_GELU) {
-        const float* b1 = p.B1 + (size_t)col * p.K;
+        const float* b1 = p.B1 + w0 + (size_t)col * p.K;
         for (int k = 0; k < p.K; ++k) s1 += a[k] * b1[k];
         s0 = gelu_dot(s0, s1);
     } else if (p.epilogue == EPI_RELU) {
@@ -373,6 +376,22 @@ bool fast_path_ok(const GemmProblem& p) {
     return p.K % 32 == 0 && (bits & 15) == 0;
 }
 
+}  // namespace
+
+bool expert_gemm_grouped_ok(const GemmProblem& p, size_t weight_stride) {
+    return fast_path_ok(p) && weight_stride % 4 == 0;
+}
+
+hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t weight_stride, const int* row_expert,
+                                                int rows, hipStream_t stream) {
+    if (rows <= 0) return hipSuccess;
+    const size_t n = (size_t)rows * p.N;
+    expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows, weight_stride, row_expert);
+    return hipGetLastError();
+}
+
+namespace {
+
 constexpr int kBN = 128;
 constexpr size_t kLdsPerCu = 160 * 1024;  // the limit is raised once, to all there is; launches ask for what they use
 
@@ -382,7 +401,7 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
     if (rows <= 0) return hipSuccess;
     if (!fast_path_ok(p)) {
         const size_t n = (size_t)rows * p.N;
-        expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows);
+        expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows, 0, nullptr);
         return hipGetLastError();
     }
     const int tile = gemm_tile_rows(p.epilogue);
@@ -404,7 +423,7 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
                                       const int* sched, int max_tiles, hipStream_t stream) {
     if (max_tiles <= 0) return hipSuccess;
-    if (!fast_path_ok(p) || weight_stride % 4 != 0) return hipErrorInvalidValue;  // callers fall back per expert
+    if (!expert_gemm_grouped_ok(p, weight_stride)) return hipErrorInvalidValue;  // see launch_expert_gemm_any_shape_grouped
     const int n_col_tiles = (p.N + kBN - 1) / kBN;
     const dim3 grid((unsigned)kXcdCount * (unsigned)xcd_tile_capacity(max_tiles) * (unsigned)n_col_tiles);
     hipError_t err;

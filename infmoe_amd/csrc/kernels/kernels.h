@@ -96,6 +96,12 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream
 // B + e*weight_stride (floats).  Row tiles and their number come from launch_expert_count.
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
                                       const int* sched, int max_tiles, hipStream_t stream);
+// Whether the grouped matrix-core launch takes this problem (K a multiple of 32, 16-byte aligned
+// operands); if not, the launch below does every routed row (row r with the weights of expert
+// row_expert[r]) one output element per thread.
+bool expert_gemm_grouped_ok(const GemmProblem& p, size_t weight_stride);
+hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t weight_stride, const int* row_expert,
+                                                int rows, hipStream_t stream);
 constexpr int kGemmTileRows = 256;       // tallest row tile of the GEMM kernel
 constexpr int kGemmTileRowsGated = 128;  // ... of its two-matrix (gated) form
 inline int gemm_tile_rows(int epilogue) { return epilogue == EPI_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }

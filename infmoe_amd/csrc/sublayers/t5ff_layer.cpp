@@ -199,6 +199,13 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     g2.epilogue = EPI_RESIDUAL;
     const bool skinny = skinnyMaxRows(T) > 0;
     if (g.afterNorm) INFMOE_HIP(hipEventRecord(g.afterNorm, g.stream));
+    if (!expert_gemm_grouped_ok(g1, stride) || !expert_gemm_grouped_ok(g2, stride)) {
+        // sizes the matrix-core kernel does not take (d or h not a multiple of 32)
+        INFMOE_HIP(launch_expert_gemm_any_shape_grouped(g1, stride, g.rowExpert, T, g.stream));
+        if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, g.stream));
+        INFMOE_HIP(launch_expert_gemm_any_shape_grouped(g2, stride, g.rowExpert, T, g.stream));
+        return INFMOE_OK;
+    }
     INFMOE_HIP(launch_expert_gemm_grouped(g1, stride, g.tiles, g.sched, g.maxTiles, g.stream));
     if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g1, stride, g.count, g.offset, mExpertCount, g.stream));
     if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, g.stream));

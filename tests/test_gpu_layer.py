@@ -96,16 +96,45 @@ def test_variants_streamed_and_resident(torch_cuda, variant, norm, ffn, mc):
     plugin.terminate()
 
 
-def test_output_is_bit_identical_for_every_max_concurrency(torch_cuda):
+@pytest.mark.parametrize("variant", ["cpm_2", "base_layer"])
+def test_output_is_bit_identical_for_every_max_concurrency(torch_cuda, variant):
+    """Streamed experts run one set of launches per expert, resident ones one grouped set: same
+    arithmetic, same bits."""
     torch = torch_cuda
     shape, E, d, h = (2, 150), 5, 64, 192
     outs = []
     for mc in (1, 2, 3, 5, 9):
-        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "cpm_2", seed=8)
+        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, variant, seed=8)
         outs.append(plugin.forward(dev(torch, x.reshape(2, 150, d))).cpu().numpy())
         plugin.terminate()
     for o in outs[1:]:
         np.testing.assert_array_equal(o, outs[0])
+
+
+@pytest.mark.parametrize("d,h", [(40, 72), (30, 50)])  # multiples of 4 but not of 32; not even of 4
+@pytest.mark.parametrize("variant,ffn", [("cpm_2", "relu"), ("base_layer", "gated_gelu")])
+@pytest.mark.parametrize("mc", [2, 4])
+def test_sizes_the_matrix_core_kernels_do_not_take(torch_cuda, d, h, variant, ffn, mc):
+    shape, E = (3, 50), 4
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, variant, ffn=ffn, seed=47)
+    run_and_check(torch_cuda, plugin, x, c, g, ws, shape, variant, ffn=ffn)
+    plugin.terminate()
+
+
+def test_output_may_alias_input(torch_cuda):
+    """The input is copied into the routed buffer before anything writes the output, so a caller
+    may pass one buffer for both."""
+    torch = torch_cuda
+    shape, E, d, h = (2, 90), 4, 64, 128
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, E, "base_layer", seed=53)
+    y, ref, _, _ = run_and_check(torch, plugin, x, c, g, ws, shape, "base_layer")
+    buf = dev(torch, x.reshape(2, 90, d))
+    ws_bytes = plugin.workspace_size([2, 90, d])
+    work = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    plugin.enqueue([2, 90, d], buf.data_ptr(), buf.data_ptr(), work.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(buf.cpu().numpy().reshape(-1, d), y)
+    plugin.terminate()
 
 
 def test_decode_shape_uses_few_row_kernels_and_matches(torch_cuda):
