@@ -302,6 +302,13 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
         g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
         g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
+        if (skinnyMax > 0) {
+            // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
+            // of them, each with one tile more than its rows fill.  A decode call then launches a small
+            // grid (or none) for the matrix-core kernel instead of one sized for E experts.
+            const int tall = T / (skinnyMax + 1);
+            g.maxTiles = std::min(c.maxTiles, tall + T / mSublayer->rowTileHeight());
+        }
         if (timed) g.afterNorm = mMarks[4], g.afterGemm1 = mMarks[5];
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {
