@@ -36,6 +36,8 @@ Status MoELayer::create(MoEParams&& p, std::unique_ptr<MoELayer>* out) {
     if (p.expertCount <= 0) return fail(INFMOE_ERR_MISSING_FIELD, "expert_count must be given and positive");
     if (p.hiddenSize <= 0) return fail(INFMOE_ERR_MISSING_FIELD, "hidden_size must be given and positive");
     if (p.maxConcurrency <= 0) return fail(INFMOE_ERR_INVALID_ARGUMENT, "max_concurrency must be positive");
+    if (p.normKind != NORM_RMS && p.normKind != NORM_CENTERED) return fail(INFMOE_ERR_INVALID_ARGUMENT, "bad norm_kind %d", p.normKind);
+    if (p.ffnKind != FFN_RELU && p.ffnKind != FFN_GATED_GELU) return fail(INFMOE_ERR_INVALID_ARGUMENT, "bad ffn_kind %d", p.ffnKind);
     if (p.centroids.empty()) return fail(INFMOE_ERR_MISSING_FIELD, "expert_centroids is required");
     if (p.centroids.size() != (size_t)p.embeddingSize * p.expertCount)
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "expert_centroids has %zu floats, expected expert_count*embedding_size = %zu",

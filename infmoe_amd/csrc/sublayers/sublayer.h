@@ -9,6 +9,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <memory>
+#include <atomic>
 #include <string>
 
 #include "../kernels/kernels.h"
@@ -46,7 +47,10 @@ class MoESubLayer {
     int mHiddenSize;
     int mMaxConcurrency;
     std::string mWeightFile;
-    int mLayerTokenCount = 0;  // tokens of the whole layer call the next run() belongs to
+    // Tokens of the whole layer call the next run() belongs to (only picks between two kernels of equal
+    // results to rounding).  Clones share the sub-layer, as in the reference
+    // (plugin/MoELayerPlugin.cc:100): atomic, so that clones driven from different threads do not race.
+    std::atomic<int> mLayerTokenCount{0};
 
    public:
     MoESubLayer(int expertCount, int embeddingSize, int hiddenSize, const char* weightFile, int maxConcurrency)
@@ -86,7 +90,7 @@ class MoESubLayer {
     // Tallest row tile runGrouped wants the dispatch scan to cut an expert's rows into.
     virtual int rowTileHeight() const { return kGemmTileRows; }
     virtual Status runGrouped(const GroupedRun& g) = 0;
-    void setLayerTokenCount(int32_t tokens) { mLayerTokenCount = tokens; }
+    void setLayerTokenCount(int32_t tokens) { mLayerTokenCount.store(tokens, std::memory_order_relaxed); }
     int expertCount() const { return mExpertCount; }
 };
 

@@ -78,6 +78,10 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)expert);
     memcpy(slot + off, host, cnt * sizeof(float));
     mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
+    if (mDeviceWeights != nullptr) {  // already resident: keep the device copy in step (blocking; not a hot path)
+        char* dev = static_cast<char*>(mDeviceWeights) + slotStride() * (size_t)expert + off * sizeof(float);
+        INFMOE_HIP(hipMemcpy(dev, slot + off, cnt * sizeof(float), hipMemcpyHostToDevice));
+    }
     return INFMOE_OK;
 }
 
@@ -176,8 +180,9 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
 Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                       hipStream_t stream) {
     // outside a layer call (token count of the call unknown) the expert stands alone
-    const bool inLayer = mLayerTokenCount > 0;
-    return runOne(tokenCount, inLayer ? mLayerTokenCount : tokenCount, inLayer ? mExpertCount : 1,
+    const int layerTokens = mLayerTokenCount.load(std::memory_order_relaxed);
+    const bool inLayer = layerTokens > 0;
+    return runOne(tokenCount, inLayer ? layerTokens : tokenCount, inLayer ? mExpertCount : 1,
                   mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights, static_cast<const float*>(input),
                   static_cast<float*>(output), workspace, stream);
 }

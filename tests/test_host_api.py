@@ -188,6 +188,10 @@ def test_serialization_round_trip_and_rejects_garbage():
     assert lib.infmoe_deserialize(b"x", blob[:40], 40, C.byref(out)) == capi.ERR_INVALID_ARGUMENT
     assert lib.infmoe_deserialize(b"x", b"\0" * len(blob), len(blob), C.byref(out)) == capi.ERR_INVALID_ARGUMENT
     assert lib.infmoe_deserialize(b"x", blob[:-4], len(blob) - 4, C.byref(out)) == capi.ERR_INVALID_ARGUMENT
+    for word, value in ((6, 7), (7, -1), (12, 5)):  # norm kind, ffn kind, number of centroid floats
+        bad = np.frombuffer(blob, np.int32).copy()
+        bad[word] = value
+        assert lib.infmoe_deserialize(b"x", bad.tobytes(), bad.nbytes, C.byref(out)) != capi.OK
 
 
 def test_binding_marshals_reference_field_names():
