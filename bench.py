@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # benchmark scaled by what the same counters read for the row-copy kernels of known size
 # (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt).  Counters cannot be read from inside a run.
-MEASURED_TRAFFIC_BYTES = {"c2": 5.70e9, "c5": 4.04e9}
+MEASURED_TRAFFIC_BYTES = {"c2": 5.74e9, "c5": 4.04e9}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
