@@ -143,10 +143,14 @@ int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stat
  * [4] first expert GEMM (activation fused), [5] second expert GEMM (residual fused),
  * [6] gather / mix.  Phases 3-5 are only separated when all experts are resident (otherwise the
  * whole streamed expert loop is reported in [4]).  `ms` holds INFMOE_N_PHASES floats.
+ * `enable` is the number of most recent calls whose marks are kept (0 = off, 1 = the last call, up
+ * to 4096); infmoe_timing_history returns those of the last min(max_calls, kept) calls, oldest
+ * first, INFMOE_N_PHASES floats per call, and their number in *n_calls.
  */
 #define INFMOE_N_PHASES 7
 int32_t infmoe_set_timing(infmoe_plugin* p, int32_t enable);
 int32_t infmoe_last_timing(infmoe_plugin* p, float* ms);
+int32_t infmoe_timing_history(infmoe_plugin* p, float* ms, int32_t max_calls, int32_t* n_calls);
 
 /* Replaces getSerializationSize / serialize / deserializePlugin (plugin/MoELayerPlugin.cc:104-143,418-458).
  * A versioned little-endian format of this library's own; expert weights are not serialised,

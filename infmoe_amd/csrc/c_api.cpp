@@ -188,7 +188,7 @@ int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stat
 int32_t infmoe_set_timing(infmoe_plugin* p, int32_t enable) {
     return guarded([&]() -> int32_t {
         INFMOE_TRY(check(p));
-        return p->layer->setTiming(enable != 0);
+        return p->layer->setTiming(enable);
     });
 }
 
@@ -197,6 +197,16 @@ int32_t infmoe_last_timing(infmoe_plugin* p, float* ms) {
         INFMOE_TRY(check(p));
         if (ms == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null output pointer");
         return p->layer->lastTiming(ms);
+    });
+}
+
+int32_t infmoe_timing_history(infmoe_plugin* p, float* ms, int32_t max_calls, int32_t* n_calls) {
+    return guarded([&]() -> int32_t {
+        INFMOE_TRY(check(p));
+        int n = 0;
+        INFMOE_TRY(p->layer->timingHistory(ms, max_calls, &n));
+        if (n_calls) *n_calls = n;
+        return INFMOE_OK;
     });
 }
 

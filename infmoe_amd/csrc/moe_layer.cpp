@@ -245,7 +245,8 @@ Status MoELayer::terminate() {
     }
     for (auto e : mMarks) (void)hipEventDestroy(e);
     mMarks.clear();
-    mTimed = false;
+    mTimedCalls = 0;
+    mTimingDepth = 0;
     if (mFork) (void)hipEventDestroy(mFork);
     if (mRoutingDone) (void)hipEventDestroy(mRoutingDone);
     mFork = mRoutingDone = nullptr;
@@ -276,8 +277,9 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     mSublayer->setLayerTokenCount(T);
 
     const bool timed = mTiming && !mMarks.empty();
+    hipEvent_t* marks = timed ? &mMarks[(size_t)(mTimedCalls % mTimingDepth) * (INFMOE_N_PHASES + 1)] : nullptr;
     auto mark = [&](int i) -> Status {
-        if (timed) INFMOE_HIP(hipEventRecord(mMarks[i], stream));
+        if (timed) INFMOE_HIP(hipEventRecord(marks[i], stream));
         return INFMOE_OK;
     };
     INFMOE_TRY(mark(0));
@@ -311,7 +313,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
             const int tall = T / (skinnyMax + 1);
             g.maxTiles = std::min(c.maxTiles, tall + T / mSublayer->rowTileHeight());
         }
-        if (timed) g.afterNorm = mMarks[4], g.afterGemm1 = mMarks[5];
+        if (timed) g.afterNorm = marks[4], g.afterGemm1 = marks[5];
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {
         INFMOE_TRY(mark(4));
@@ -327,29 +329,46 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     else
         INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream));
     INFMOE_TRY(mark(7));
-    mTimed = timed;
+    if (timed) ++mTimedCalls;
     return INFMOE_OK;
 }
 
-Status MoELayer::setTiming(bool enable) {
-    if (enable && mMarks.empty()) {
-        mMarks.resize(INFMOE_N_PHASES + 1);
+Status MoELayer::setTiming(int depth) {
+    if (depth < 0 || depth > 4096) return fail(INFMOE_ERR_INVALID_ARGUMENT, "timing depth must be 0..4096");
+    if (depth != mTimingDepth) {
+        for (auto e : mMarks) (void)hipEventDestroy(e);
+        mMarks.assign((size_t)depth * (INFMOE_N_PHASES + 1), nullptr);
         for (auto& e : mMarks) INFMOE_HIP(hipEventCreate(&e));
+        mTimingDepth = depth;
     }
-    mTiming = enable;
-    mTimed = false;
+    mTiming = depth > 0;
+    mTimedCalls = 0;
+    return INFMOE_OK;
+}
+
+Status MoELayer::timingHistory(float* ms, int maxCalls, int* nCalls) {
+    if (ms == nullptr || nCalls == nullptr || maxCalls < 0) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null output");
+    const long long kept = std::min<long long>(mTimedCalls, mTimingDepth);
+    const int n = (int)std::min<long long>(kept, maxCalls);
+    *nCalls = n;
+    for (int j = 0; j < n; ++j) {  // oldest of the n first
+        const long long call = mTimedCalls - n + j;
+        hipEvent_t* marks = &mMarks[(size_t)(call % mTimingDepth) * (INFMOE_N_PHASES + 1)];
+        INFMOE_HIP(hipEventSynchronize(marks[INFMOE_N_PHASES]));
+        for (int i = 0; i < INFMOE_N_PHASES; ++i) {
+            float* out = ms + (size_t)j * INFMOE_N_PHASES + i;
+            *out = 0.f;
+            // an Identity sub-layer or a streamed expert loop leaves some marks unrecorded
+            if (hipEventElapsedTime(out, marks[i], marks[i + 1]) != hipSuccess) *out = 0.f;
+        }
+    }
     return INFMOE_OK;
 }
 
 Status MoELayer::lastTiming(float* ms) {
-    if (!mTimed) return fail(INFMOE_ERR_STATE, "no timed enqueue to report (infmoe_set_timing, then infmoe_enqueue)");
-    INFMOE_HIP(hipEventSynchronize(mMarks[INFMOE_N_PHASES]));
-    for (int i = 0; i < INFMOE_N_PHASES; ++i) {
-        ms[i] = 0.f;
-        // an Identity sub-layer or a streamed expert loop leaves some marks unrecorded in this call
-        if (hipEventElapsedTime(&ms[i], mMarks[i], mMarks[i + 1]) != hipSuccess) ms[i] = 0.f;
-    }
-    return INFMOE_OK;
+    if (mTimedCalls == 0) return fail(INFMOE_ERR_STATE, "no timed enqueue to report (infmoe_set_timing, then infmoe_enqueue)");
+    int n = 0;
+    return timingHistory(ms, 1, &n);
 }
 
 // Experts streamed through max_concurrency device slots (plugin/MoELayerPlugin.cc:360-402).

@@ -44,8 +44,9 @@ class MoELayer {
     Status terminate();                                                        // :203-237
     Status setScoreBias(const float* host);
     Status lastRouting(int32_t* countHost, int32_t* statsHost);
-    Status setTiming(bool enable);
+    Status setTiming(int depth);  // 0: off; n: keep the phase marks of the last n calls
     Status lastTiming(float* ms);
+    Status timingHistory(float* ms, int maxCalls, int* nCalls);
 
     Status serializationSize(size_t* bytes) const;
     Status serialize(void* buffer, size_t bytes) const;
@@ -79,8 +80,10 @@ class MoELayer {
     std::vector<hipStream_t> mComputeStreams;
     std::vector<hipEvent_t> mCopyDone, mComputeDone, mJoin;
     hipEvent_t mFork = nullptr, mRoutingDone = nullptr;
-    bool mTiming = false, mTimed = false;
-    std::vector<hipEvent_t> mMarks;  // INFMOE_N_PHASES + 1 phase boundaries
+    bool mTiming = false;
+    int mTimingDepth = 0;            // calls whose marks are kept
+    long long mTimedCalls = 0;       // timed calls since timing was switched on
+    std::vector<hipEvent_t> mMarks;  // mTimingDepth sets of INFMOE_N_PHASES + 1 phase boundaries
 };
 
 }  // namespace infmoe

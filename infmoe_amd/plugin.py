@@ -73,8 +73,17 @@ class Plugin:
 
     PHASES = ("gating", "count_sort", "scatter", "expert_norm", "expert_gemm1", "expert_gemm2", "gather")
 
-    def set_timing(self, enable: bool) -> None:
+    def set_timing(self, enable) -> None:
+        """False / 0: off.  True / 1: keep the phase marks of the last call.  n: of the last n calls."""
         capi.check(self._lib.infmoe_set_timing(self._h, int(enable)))
+
+    def timing_history(self, max_calls: int) -> list:
+        """Phase times (ms) of the last min(max_calls, kept) calls, oldest first."""
+        n = len(self.PHASES)
+        ms = (C.c_float * (n * max_calls))()
+        got = C.c_int32(0)
+        capi.check(self._lib.infmoe_timing_history(self._h, ms, max_calls, C.byref(got)))
+        return [dict(zip(self.PHASES, ms[i * n:(i + 1) * n])) for i in range(got.value)]
 
     def last_timing(self) -> dict:
         ms = (C.c_float * len(self.PHASES))()

@@ -276,3 +276,28 @@ def test_layer_can_be_captured_in_a_graph_and_replayed(torch_cuda):
             assert torch.equal(yout, eager[k]), f"replay {rep}/{k} differs from the eager result"
             assert torch.equal(plugin.forward(v), eager[k])  # eager work between replays
     plugin.terminate()
+
+
+def test_phase_timing_keeps_the_last_calls(torch_cuda):
+    torch = torch_cuda
+    shape, E, d, h = (2, 64), 4, 64, 128
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, E, "cpm_2", seed=59)
+    xd = dev(torch, x.reshape(2, 64, d))
+    with pytest.raises(RuntimeError):
+        plugin.last_timing()  # nothing timed yet
+    plugin.set_timing(3)
+    for _ in range(5):
+        plugin.forward(xd)
+    hist = plugin.timing_history(10)
+    assert len(hist) == 3  # the last three of five calls
+    for phases in hist:
+        assert set(phases) == set(plugin.PHASES)
+        assert all(v >= 0.0 for v in phases.values())
+        assert phases["expert_gemm1"] > 0.0 and phases["gating"] > 0.0
+    assert plugin.last_timing() == hist[-1]
+    assert len(plugin.timing_history(2)) == 2
+    plugin.set_timing(False)
+    plugin.forward(xd)
+    with pytest.raises(RuntimeError):
+        plugin.last_timing()
+    plugin.terminate()
