@@ -301,3 +301,13 @@ def test_phase_timing_keeps_the_last_calls(torch_cuda):
     with pytest.raises(RuntimeError):
         plugin.last_timing()
     plugin.terminate()
+
+
+@pytest.mark.parametrize("E,mc", [(130, 130), (130, 3), (64, 64)])
+def test_many_experts(torch_cuda, E, mc):
+    """More experts than one gating pass scores (128), most of them with a handful of rows."""
+    shape, d, h = (7, 100), 64, 96
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "cpm_2", seed=61)
+    y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "cpm_2")
+    assert count.sum() == 700 and (count > 0).sum() > E // 2
+    plugin.terminate()
