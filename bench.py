@@ -40,6 +40,20 @@ CONFIGS = {
 }
 
 
+def zipf_score_bias(x, centroids, s=1.2, iters=30):
+    """Input synthesis for the skewed workload: a per-expert additive score bias such that the
+    top-1 counts follow p_e ~ (e+1)^-s (fixed-point iteration on the host; not a reference attribute)."""
+    aff = np.asarray(x, np.float64) @ np.asarray(centroids, np.float64).T
+    T, E = aff.shape
+    target = np.arange(1, E + 1) ** (-float(s))
+    target = target / target.sum()
+    bias = np.zeros(E)
+    for _ in range(iters):
+        p = np.bincount(np.argmax(aff + bias, axis=1), minlength=E) / T
+        bias += 0.5 * (np.log(target) - np.log(np.maximum(p, 0.5 / T)))
+    return bias.astype(np.float32)
+
+
 def build_layer(torch, cfg, seed=0, keep_host=True, replicate=False):
     """Synthetic tensors drawn on the GPU (fixed seed), expert weights handed to the library by
     host pointer, as a caller holding an npz in memory would."""
@@ -80,8 +94,7 @@ def build_layer(torch, cfg, seed=0, keep_host=True, replicate=False):
             slots.append(slot)
     bias = None
     if cfg["zipf"]:
-        from oracle import moe_oracle as O  # harness-side calibration of the skew only
-        bias = O.zipf_score_bias(x.cpu().numpy(), cent.cpu().numpy(), s=1.2)
+        bias = zipf_score_bias(x.cpu().numpy(), cent.cpu().numpy(), s=1.2)
         plugin.set_score_bias(bias)
     plugin.configure([B, S, d])
     plugin.initialize()
