@@ -377,7 +377,8 @@ Status MoELayer::lastTiming(float* ms) {
 //   copy stream:   [wait: expert k-mc done] copy expert k into slot k % mc, signal copyDone[k]
 //   compute k%n:   [wait: copyDone[k]] run expert k from its slot,          signal computeDone[k]
 // so up to mc-1 experts are prefetched while one computes (the reference prefetches one), and
-// max_concurrency = 1 degenerates to copy, compute, copy, ... with no overlap.
+// max_concurrency = 1 degenerates to copy, compute, copy, ... with no overlap.  Experts run in
+// descending order of their row counts.
 Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
     const size_t routingInts = (size_t)2 * E + 1 + 4;
@@ -391,9 +392,17 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     INFMOE_HIP(hipEventRecord(mFork, stream));
     INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
     for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
+    // Empty experts are skipped (:361-363,383-384).  The reference takes the others in ascending
+    // index; here the ones with most rows go first (stable, so equal counts stay ascending): every
+    // expert costs the same copy, and the compute that nothing can hide is the last expert's, so it
+    // should be the shortest.  Rows of different experts are disjoint: the order cannot change a bit.
+    std::vector<int> order;
+    order.reserve(E);
+    for (int e = 0; e < E; ++e)
+        if (count[e] > 0) order.push_back(e);
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return count[a] > count[b]; });
     int k = 0;
-    for (int e = 0; e < E; ++e) {  // ascending, empty experts skipped (:361-363,383-384)
-        if (count[e] == 0) continue;
+    for (const int e : order) {
         const int slot = k % mc;
         char* slotPtr = c.slots + c.slotStride * (size_t)slot;
         if (k >= mc) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[k - mc], 0));
