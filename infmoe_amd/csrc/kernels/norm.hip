@@ -4,7 +4,9 @@
 //   rms:      gamma * x * rsqrt(mean(x^2) + eps)                    (README.md:115)
 // One wave per row.  The row is read once into registers when it is at most 8192 floats (two
 // exact passes for the centered form: mean, then variance about the mean, instead of the
-// reference's Welford merge) and re-read from cache otherwise.  For the grouped expert launch
+// reference's Welford merge) and re-read from cache otherwise.  The register array is sized for the
+// row (2048, 4096 or 8192 floats): with the largest size for every row only three waves fit a SIMD,
+// and 4096 rows then run as one full generation of workgroups plus a third of one.  For the grouped expert launch
 // every routed row picks the gamma of its own expert.
 #include <hip/hip_runtime.h>
 
@@ -15,7 +17,7 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
-constexpr int kRegVec = 32;  // float4 per lane held in registers -> rows up to 64*32*4 = 8192 floats
+constexpr int kMaxRegVec = 32;  // float4 per lane held in registers -> rows up to 64*32*4 = 8192 floats
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -23,7 +25,8 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-template <bool VEC>
+// RV: float4 per lane held in registers (rows of up to 256 * RV floats take the one-pass form)
+template <bool VEC, int RV>
 __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                             int rows, int d, const float* __restrict__ gamma_base,
                                                             size_t gamma_stride, const int* __restrict__ row_expert,
@@ -36,24 +39,24 @@ __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ 
     const float* g = gamma_base + (row_expert ? (size_t)row_expert[r] * gamma_stride : 0);
     const float inv_d = 1.0f / (float)d;
 
-    if (VEC && d <= 64 * 4 * kRegVec) {
+    if (VEC && d <= 64 * 4 * RV) {
         const int n4 = d >> 2;
-        v4f v[kRegVec];
+        v4f v[RV];
         float s = 0.f;
 #pragma unroll
-        for (int j = 0; j < kRegVec; ++j) {
+        for (int j = 0; j < RV; ++j) {
             const int k = lane + 64 * j;
             v[j] = (k < n4) ? reinterpret_cast<const v4f*>(x)[k] : v4f{0.f, 0.f, 0.f, 0.f};
         }
         float mu = 0.f;
         if (norm_kind == NORM_CENTERED) {
 #pragma unroll
-            for (int j = 0; j < kRegVec; ++j) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+            for (int j = 0; j < RV; ++j) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
             mu = wave_sum(s) * inv_d;
         }
         float q = 0.f;
 #pragma unroll
-        for (int j = 0; j < kRegVec; ++j) {
+        for (int j = 0; j < RV; ++j) {
             const int k = lane + 64 * j;
             if (k < n4) {
                 const v4f c = v[j] - mu;
@@ -62,7 +65,7 @@ __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ 
         }
         const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_d + kNormEps);
 #pragma unroll
-        for (int j = 0; j < kRegVec; ++j) {
+        for (int j = 0; j < RV; ++j) {
             const int k = lane + 64 * j;
             if (k < n4) reinterpret_cast<v4f*>(y)[k] = reinterpret_cast<const v4f*>(g)[k] * ((v[j] - mu) * rstd);
         }
@@ -92,12 +95,17 @@ hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const f
     const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in) |
                            reinterpret_cast<uintptr_t>(gamma_base)) & 15) == 0 &&
                          (gamma_stride % 4 == 0);
-    if (d % 4 == 0 && aligned)
-        row_norm_kernel<true><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert,
-                                                             norm_kind);
-    else
-        row_norm_kernel<false><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert,
-                                                              norm_kind);
+#define INFMOE_NORM(V, RV)                                                                                        \
+    row_norm_kernel<V, RV><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert, \
+                                                          norm_kind)
+    if (d % 4 == 0 && aligned) {
+        if (d <= 2048) INFMOE_NORM(true, 8);
+        else if (d <= 4096) INFMOE_NORM(true, 16);
+        else INFMOE_NORM(true, kMaxRegVec);
+    } else {
+        INFMOE_NORM(false, 1);
+    }
+#undef INFMOE_NORM
     return hipGetLastError();
 }
 
