@@ -167,10 +167,19 @@ __device__ __forceinline__ void rank_body(int T, int E, const int* __restrict__ 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const int base = blockIdx.x * kCountBlockTokens;
+    // all of this thread's assignments are fetched before the first barrier: inside the loop every
+    // load would cost a memory round trip of its own
+    int chosen[kPerThread];
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+        const int t = base + j * kThreads + threadIdx.x;
+        chosen[j] = t < T ? min(max(sel[t], 0), E - 1) : -1;
+    }
+#pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
         const int t = base + j * kThreads + threadIdx.x;  // token order == (j, wave, lane) order
         const bool valid = t < T;
-        const int e = valid ? min(max(sel[t], 0), E - 1) : -1;
+        const int e = chosen[j];
         // rank among the lanes of this wave that chose the same expert
         int rank = 0, cnt = 0;
         bool leader = false;
@@ -186,15 +195,18 @@ __device__ __forceinline__ void rank_body(int T, int E, const int* __restrict__ 
             }
             todo &= ~same;
         }
-        // waves take turns so that earlier tokens get lower rows
+        // waves take turns so that earlier tokens get lower rows; inside a wave every lane has read
+        // its expert's running count before the leaders advance it (LDS operations of one wave
+        // complete in order), so one barrier per turn is enough
         for (int w = 0; w < kThreads / 64; ++w) {
-            if (wave == w && valid) {
-                const int r = s_run[e] + rank;
-                pos[r] = t;
-                if (row_expert != nullptr) row_expert[r] = e;
+            if (wave == w) {
+                const int r = valid ? s_run[e] + rank : 0;
+                if (valid) {
+                    pos[r] = t;
+                    if (row_expert != nullptr) row_expert[r] = e;
+                }
+                if (leader) s_run[e] = r - rank + cnt;
             }
-            __syncthreads();
-            if (wave == w && leader) s_run[e] += cnt;
             __syncthreads();
         }
     }
