@@ -7,7 +7,7 @@
 //      row tiles of the grouped expert launch,
 //   3. stable ranking: token t goes to row offset[e] + (tokens of e in earlier blocks) +
 //      (tokens of e earlier in this block).  The rank inside a block is built from wave ballots
-//      in token order, so the permutation does not depend on the order atomics retire in and is
+//      (one per bit of the expert index) in token order, so the permutation does not depend on the order atomics retire in and is
 //      bit-identical to the reference's sequential counting sort.
 // and the row-copy kernels batch_scatter_feature_and_weight_kernel / batch_gather_kernel /
 // fused_batch_mix_and_gather_kernel (plugin/cuda/moe.cu:89-127) by wave-per-row copies with
@@ -167,6 +167,7 @@ __device__ __forceinline__ void rank_body(int T, int E, const int* __restrict__ 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const int base = blockIdx.x * kCountBlockTokens;
+    const int index_bits = E > 1 ? 32 - __clz(E - 1) : 0;
     // all of this thread's assignments are fetched before the first barrier: inside the loop every
     // load would cost a memory round trip of its own
     int chosen[kPerThread];
@@ -180,21 +181,18 @@ __device__ __forceinline__ void rank_body(int T, int E, const int* __restrict__ 
         const int t = base + j * kThreads + threadIdx.x;  // token order == (j, wave, lane) order
         const bool valid = t < T;
         const int e = chosen[j];
-        // rank among the lanes of this wave that chose the same expert
-        int rank = 0, cnt = 0;
-        bool leader = false;
-        unsigned long long todo = __ballot(valid);
-        while (todo) {
-            const int first = __ffsll((long long)todo) - 1;
-            const int ef = __shfl(e, first);
-            const unsigned long long same = __ballot(valid && e == ef);
-            if (e == ef) {
-                rank = __popcll(same & below);
-                cnt = __popcll(same);
-                leader = (lane == first);
-            }
-            todo &= ~same;
+        // Lanes of this wave that chose the same expert: one ballot per bit of the expert index
+        // (a lane keeps the lanes that agree with it on every bit), instead of one round per distinct
+        // expert in the wave.
+        unsigned long long same = __ballot(valid);
+        for (int bit = 0; bit < index_bits; ++bit) {
+            const bool set = (e >> bit) & 1;
+            const unsigned long long m = __ballot(valid && set);
+            same &= set ? m : ~m;
         }
+        const int rank = __popcll(same & below);  // earlier lanes of the group
+        const int cnt = __popcll(same);
+        const bool leader = valid && (same & below) == 0;
         // waves take turns so that earlier tokens get lower rows; inside a wave every lane has read
         // its expert's running count before the leaders advance it (LDS operations of one wave
         // complete in order), so one barrier per turn is enough
