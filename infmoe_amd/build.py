@@ -17,10 +17,15 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libinfmoe.so")
 
 SOURCES = [
-    "kernels/gating.hip",
     "kernels/dispatch.hip",
     "kernels/norm.hip",
+    # the four instantiations of the matrix-core expert kernel first: they take longest
+    "kernels/expert_gemm_grouped.hip",
+    "kernels/expert_gemm_one.hip",
+    "kernels/expert_gemm_grouped_gated.hip",
+    "kernels/expert_gemm_one_gated.hip",
     "kernels/expert_gemm.hip",
+    "kernels/gating.hip",
     "kernels/expert_skinny.hip",
     "sublayers/t5ff_layer.cpp",
     "npz_reader.cpp",

@@ -5,6 +5,12 @@
 
 namespace infmoe {
 
+// plugin/cuda/ops/gelu.cu:8-15
+__device__ __forceinline__ float gelu_dot(float a, float b) {
+    const float cdf = 0.5f * (1.0f + tanhf(a * (0.035677408136300125f * a * a + 0.7978845608028654f)));
+    return a * cdf * b;
+}
+
 // plugin/cuda/common.cuh:24-27
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 

@@ -1,0 +1,383 @@
+// FP32 matrix-core GEMM of the T5 feed-forward expert for gfx950: device code.
+// Included by the translation units that instantiate one kernel each (the tile body exists in some
+// seventy shapes per kernel, so they compile side by side).
+//
+// Replaces the three cublasSgemm_v2 calls, the thrust gelu*mul pass and the device-to-device
+// residual copy of T5FFLayer::run (plugin/sublayers/T5FFLayer.cc:112-138, plugin/cuda/ops/gelu.cu:7-25):
+//     C[rows][N] = epilogue(A[rows][K] * B[N][K]^T)
+// with both operands K-contiguous (activations row-major, weights in torch Linear layout), which
+// is the "TN" form the FP32 matrix-core instructions want: a lane feeds one float of an A row and
+// one float of a B row per instruction.  The work is done by v_mfma_f32_32x32x2_f32, which on this
+// part sustains 99% of the 157 TFLOP/s peak from one wave per SIMD where v_mfma_f32_16x16x4_f32
+// tops out at 79% (measured with register-only loops); the 16x16x4 form is kept for one 16-row
+// block at the bottom of a tile so that row counts are padded to 16, not 32.
+//
+// Tiling.  The weights are the big operand (335 MB per expert at d=4096, h=10240) and each weight
+// element is reused only `rows` times, so a workgroup covers ALL rows of its expert (up to 256) x
+// BN weight rows: every weight byte is fetched from HBM once.  Token counts per expert vary, so the
+// tile height is a run-time multiple of 16 rows (NMB of them: NMB/2 blocks of 32 rows plus one of
+// 16 when NMB is odd); the body is instantiated for NMB = 1..16 and selected per workgroup, which
+// wastes at most 15 padded rows per expert instead of up to a whole fixed-height tile.  The 4
+// waves of a workgroup split the BN = 128 columns, 32 each, and keep the accumulators of all row
+// blocks in registers.
+//
+// Pipeline.  K advances in steps of 32 floats.  While the matrix core works on step s from one half
+// of a double-buffered LDS tile, the global loads of step s+2 go into registers and the registers
+// holding step s+1 are written to the other half; one barrier per step.  These memory operations
+// are not issued in bursts before and after the MFMAs (that left the matrix core idle a quarter of
+// the time) but dealt out a few at a time between small groups of MFMAs.  LDS rows are padded to 36 floats so that the 16-byte
+// operand reads of the lanes of a block hit distinct banks.  Inside an 8-float (32x32x2) or 16-float
+// (16x16x4) chunk the k order is permuted identically for A and B (lane group q supplies floats
+// 4q..4q+3 over four instructions), which a dot product does not see and which lets every operand
+// read be a ds_read_b128.
+//
+// Grouped launch.  One launch covers every expert: row tiles come from the device-side table built
+// by the dispatch scan, so no token count ever travels to the host.  Workgroup ids are dealt
+// round-robin to the 8 XCDs by the hardware; the id -> tile map undoes that so each XCD works
+// through a contiguous run of (expert, column tile) pairs and the activations of an expert stay
+// in one XCD's L2.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "device_math.h"
+#include "expert_gemm_parts.h"
+#include "kernels.h"
+
+namespace infmoe {
+namespace {
+
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kMaxMb64 = kGemmMaxUnits64;
+constexpr int kThreads = kGemmThreads;
+
+// f(integral_constant<int, I>) for I in [I0, N): an unrolled loop whose index is a constant expression
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// One output tile: `rows` (<= 16*NMB + 4*G4) rows of A against BN rows of B (and of B1 when GATED).
+// BK: floats of K per pipeline step (32 or 64).
+// G4: groups of 4 rows below the 16-row units, on v_mfma_f32_4x4x1_16b_f32 (16 blocks of 4x4 per
+// instruction: 8 blocks cover the wave's 32 columns, the two halves of the wave take the two float4 of
+// an 8-k group and their sums meet in the epilogue).  The instruction takes the B operand exactly as
+// the 32x32x2 form holds it (lane -> column lane % 32, float4 lane / 32), so a group costs one more
+// LDS read per k group and four short instructions: rows are padded to 4, not to 16.
+template <int NMB, int G4, int BN, bool GATED, int BK>
+__device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const float* __restrict__ R,
+                                          float* __restrict__ C, int rows, const float* __restrict__ B0,
+                                          const float* __restrict__ B1, int n0, int N, int K, int epilogue,
+                                          float* __restrict__ smem, int a_alloc_rows) {
+    static_assert(BN == 128, "each of the 4 waves owns one 32-column block");
+    constexpr int NB = GATED ? 2 : 1;         // weight matrices
+    constexpr int N32 = NMB / 2;              // 32-row blocks (v_mfma_f32_32x32x2_f32)
+    constexpr bool T16 = (NMB & 1) != 0;      // one trailing 16-row block (v_mfma_f32_16x16x4_f32)
+    constexpr int LDK = BK + 4;               // padded LDS row (floats)
+    constexpr int KH = BK / 32;               // 32-float halves of a step's row
+    static_assert(G4 == 0 || (!GATED && NMB >= 2), "row groups of 4 ride on the 32x32x2 slots");
+    constexpr int TAIL0 = NMB * 16;           // first row of the 4-row groups
+    constexpr int A_ROWS = NMB * 16 + 4 * G4;
+    constexpr int A_LOADS = ((A_ROWS + 31) / 32) * KH;  // float4 per thread per step: KH per 32-row slab
+    constexpr int B_LOADS = (BN / 32) * KH;
+    constexpr int NV = A_LOADS + NB * B_LOADS;   // global loads (and LDS writes) per thread per step
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i32 = lane & 31, kh = lane >> 5;  // 32x32x2: row / column fed, which float4 of 8 k
+    const int i16 = lane & 15, kq = lane >> 4;  // 16x16x4: row / column fed, which float4 of 16 k
+    const int ld_row = tid >> 3, ld_c4 = tid & 7;  // this thread's (row, float4) inside a 32-row slab
+
+    float* As = smem;                                   // [2][a_alloc_rows][LDK]
+    float* Bs = smem + 2 * (size_t)a_alloc_rows * LDK;  // [2][NB*BN][LDK]
+    const size_t a_buf = (size_t)a_alloc_rows * LDK, b_buf = (size_t)NB * BN * LDK;
+
+    v16f acc32[NB][N32 > 0 ? N32 : 1];
+    v4f acc16[NB][2];
+    v4f acc4[G4 > 0 ? G4 : 1];
+#pragma unroll
+    for (int q = 0; q < (G4 > 0 ? G4 : 1); ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < NB; ++m) {
+#pragma unroll
+        for (int mb = 0; mb < (N32 > 0 ? N32 : 1); ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc32[m][mb][r] = 0.f;
+        acc16[m][0] = v4f{0.f, 0.f, 0.f, 0.f};
+        acc16[m][1] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // Global addresses are a wave-uniform base (kept in scalar registers and advanced along K) plus a
+    // 32-bit per-thread byte offset, so a load needs no 64-bit vector arithmetic.  Rows past the end
+    // are clamped: their products land in accumulator rows / columns that are never stored.
+    const char* a_base = reinterpret_cast<const char*>(A);
+    const char* b_base[NB];
+    b_base[0] = reinterpret_cast<const char*>(B0 + (size_t)n0 * K);
+    if (GATED) b_base[NB - 1] = reinterpret_cast<const char*>(B1 + (size_t)n0 * K);
+    unsigned a_off[A_LOADS], b_off[B_LOADS];
+#pragma unroll
+    for (int p = 0; p < A_LOADS; ++p)  // item p: slab p / KH, half p % KH
+        a_off[p] = ((unsigned)min((p / KH) * 32 + ld_row, rows - 1) * (unsigned)K + 32u * (p % KH) + 4u * ld_c4) * 4u;
+#pragma unroll
+    for (int p = 0; p < B_LOADS; ++p)
+        b_off[p] = ((unsigned)min((p / KH) * 32 + ld_row, N - 1 - n0) * (unsigned)K + 32u * (p % KH) + 4u * ld_c4) * 4u;
+
+    // Two register sets: global loads run two K steps ahead of the matrix core, which covers the
+    // latency of an HBM miss (every weight load is one) with two steps of MFMA work.
+    v4f ra[2][A_LOADS], rb[2][NB][B_LOADS];
+    // item L of the global loads of the step starting at k0 (K % BK == 0 on this path), into set P
+    auto gload = [&](auto setc, auto lc, int k0) {
+        constexpr int P = decltype(setc)::value, L = decltype(lc)::value;
+        if constexpr (L < A_LOADS) {
+            ra[P][L] = *reinterpret_cast<const v4f*>(a_base + (size_t)k0 * 4 + a_off[L]);
+        } else {
+            constexpr int M = (L - A_LOADS) / B_LOADS, Q = (L - A_LOADS) % B_LOADS;
+            rb[P][M][Q] = *reinterpret_cast<const v4f*>(b_base[M] + (size_t)k0 * 4 + b_off[Q]);
+        }
+    };
+    // item L of register set P into LDS buffer BUF
+    auto lstore = [&](auto setc, auto lc, auto bufc) {
+        constexpr int P = decltype(setc)::value, L = decltype(lc)::value, BUF = decltype(bufc)::value;
+        if constexpr (L < A_LOADS) {
+            *reinterpret_cast<v4f*>(As + BUF * a_buf + ((L / KH) * 32 + ld_row) * LDK + 32 * (L % KH) + 4 * ld_c4) = ra[P][L];
+        } else {
+            constexpr int M = (L - A_LOADS) / B_LOADS, Q = (L - A_LOADS) % B_LOADS;
+            *reinterpret_cast<v4f*>(Bs + BUF * b_buf + (M * BN + (Q / KH) * 32 + ld_row) * LDK + 32 * (Q % KH) + 4 * ld_c4) =
+                rb[P][M][Q];
+        }
+    };
+
+    // MFMA operands, double-buffered by k group so that the reads of group g+1 fly under the MFMAs of g
+    v4f af32[2][N32 > 0 ? N32 : 1], bf32[2][NB];  // 32x32x2: 8-k groups
+    v4f af16[2], bf16[2][NB][2];                  // 16x16x4: 16-k groups
+    v4f af4[2][G4 > 0 ? G4 : 1];                  // 4x4x1: the 8-k groups of the 32x32x2 form, row lane % 4
+    const float* a4 = As + (TAIL0 + (lane & 3)) * LDK + 4 * kh;
+    const float* a32 = As + i32 * LDK + 4 * kh;
+    const float* b32 = Bs + (wave * 32 + i32) * LDK + 4 * kh;
+    const float* a16 = As + (32 * N32 + i16) * LDK + 4 * kq;
+    const float* b16 = Bs + (wave * 32 + i16) * LDK + 4 * kq;
+    // operand q of 8-k group g: q < NB weights, then the 32-row blocks, then the 4-row groups
+    auto read32 = [&](auto bufc, auto gc, auto qc) {
+        constexpr int BUF = decltype(bufc)::value, G = decltype(gc)::value, Q = decltype(qc)::value;
+        if constexpr (Q < NB)
+            bf32[G & 1][Q] = *reinterpret_cast<const v4f*>(b32 + BUF * b_buf + Q * BN * LDK + 8 * G);
+        else if constexpr (Q < NB + N32)
+            af32[G & 1][Q - NB] = *reinterpret_cast<const v4f*>(a32 + BUF * a_buf + 32 * (Q - NB) * LDK + 8 * G);
+        else
+            af4[G & 1][Q - NB - N32] = *reinterpret_cast<const v4f*>(a4 + BUF * a_buf + 4 * (Q - NB - N32) * LDK + 8 * G);
+    };
+    auto read16 = [&](auto bufc, auto gc, auto qc) {  // operand q of 16-k group g: 0 = rows, then weights (m, nb)
+        constexpr int BUF = decltype(bufc)::value, G = decltype(gc)::value, Q = decltype(qc)::value;
+        if constexpr (Q == 0)
+            af16[G & 1] = *reinterpret_cast<const v4f*>(a16 + BUF * a_buf + 16 * G);
+        else
+            bf16[G & 1][(Q - 1) / 2][(Q - 1) % 2] = *reinterpret_cast<const v4f*>(
+                b16 + BUF * b_buf + (((Q - 1) / 2) * BN + 16 * ((Q - 1) % 2)) * LDK + 16 * G);
+    };
+
+    // One K step = S slots.  A slot issues a few memory operations and then a handful of MFMAs,
+    // and nothing may be moved across a slot boundary, so the matrix core is fed continuously:
+    //   * the first half of the slots carries the global loads of step s + 2 (register set 1 - P),
+    //   * the second half writes register set P (step s + 1) into LDS buffer 1 - P,
+    //   * every slot group carries the LDS operand reads of the next k group.
+    // The loop over steps is unrolled by two so that P, and with it every LDS address offset and
+    // register index, is a compile-time constant.
+    constexpr int G32 = BK / 8, G16 = BK / 16;  // k groups of a step
+    constexpr int S32 = N32 > 0 ? 4 * G32 : 0, S16 = T16 ? 4 * G16 : 0, S = S32 + S16, SV = S / 2;
+    constexpr int R32 = NB + N32 + G4, R16 = 1 + 2 * NB;
+    const int nk = K / BK;
+    auto step = [&](auto setc, int s) {
+        constexpr int P = decltype(setc)::value;
+        const std::integral_constant<int, P> cur{};
+        const std::integral_constant<int, 1 - P> other{};
+        const int kload = min(s + 2, nk - 1) * BK;  // the surplus loads of the last two steps are discarded
+        if constexpr (N32 > 0)
+            static_for<0, R32>([&](auto qc) { read32(cur, std::integral_constant<int, 0>{}, qc); });
+        else
+            static_for<0, R16>([&](auto qc) { read16(cur, std::integral_constant<int, 0>{}, qc); });
+        static_for<0, S>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            if constexpr (t < SV)
+                static_for<(t * NV) / SV, ((t + 1) * NV) / SV>([&](auto lc) { gload(other, lc, kload); });
+            else
+                static_for<((t - SV) * NV) / (S - SV), ((t - SV + 1) * NV) / (S - SV)>(
+                    [&](auto lc) { lstore(cur, lc, other); });
+            if constexpr (t < S32) {
+                constexpr int g = t / 4, j = t % 4;
+                if constexpr (g < G32 - 1 && j < 3)  // a third of the next group's operands per slot
+                    static_for<0, R32>([&](auto qc) {
+                        if constexpr (decltype(qc)::value % 3 == j) read32(cur, std::integral_constant<int, g + 1>{}, qc);
+                    });
+                if constexpr (g == G32 - 1 && j < 3 && T16)
+                    static_for<0, R16>([&](auto qc) {
+                        if constexpr (decltype(qc)::value % 3 == j) read16(cur, std::integral_constant<int, 0>{}, qc);
+                    });
+#pragma unroll
+                for (int mb = 0; mb < N32; ++mb)
+#pragma unroll
+                    for (int m = 0; m < NB; ++m)
+                        acc32[m][mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(af32[g & 1][mb][j], bf32[g & 1][m][j],
+                                                                             acc32[m][mb], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < G4; ++q)
+                    acc4[q] = __builtin_amdgcn_mfma_f32_4x4x1f32(af4[g & 1][q][j], bf32[g & 1][0][j], acc4[q], 0, 0, 0);
+            } else {
+                constexpr int g = (t - S32) / 4, j = (t - S32) % 4;
+                if constexpr (g < G16 - 1 && j < 3)
+                    static_for<0, R16>([&](auto qc) {
+                        if constexpr (decltype(qc)::value % 3 == j) read16(cur, std::integral_constant<int, g + 1>{}, qc);
+                    });
+#pragma unroll
+                for (int m = 0; m < NB; ++m)
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb)
+                        acc16[m][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(af16[g & 1][j], bf16[g & 1][m][nb][j],
+                                                                             acc16[m][nb], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        __syncthreads();
+    };
+    const std::integral_constant<int, 0> set0{};
+    const std::integral_constant<int, 1> set1{};
+    static_for<0, NV>([&](auto lc) { gload(set1, lc, 0); });
+    static_for<0, NV>([&](auto lc) { lstore(set1, lc, set0); });
+    static_for<0, NV>([&](auto lc) { gload(set0, lc, min(1, nk - 1) * BK); });
+    __syncthreads();
+    for (int s = 0; s < nk; s += 2) {
+        step(set0, s);
+        if (s + 1 < nk) step(set1, s + 1);
+    }
+
+    // epilogue
+    auto emit = [&](int row, int col, float v, float v1) {
+        if (row < rows && col < N) {
+            const size_t o = (size_t)row * N + col;
+            if (GATED) {
+                v = gelu_dot(v, v1);
+            } else if (epilogue == EPI_RELU) {
+                v = fmaxf(v, 0.f);
+            } else {
+                v += R[o];
+            }
+            C[o] = v;
+        }
+    };
+    // 32x32 block: register r holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+#pragma unroll
+    for (int mb = 0; mb < N32; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            emit(32 * mb + 8 * (r / 4) + 4 * kh + (r % 4), n0 + wave * 32 + i32, acc32[0][mb][r], acc32[NB - 1][mb][r]);
+    // 16x16 block: register r holds row 4*(lane/16) + r, column lane%16
+    if (T16) {
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                emit(32 * N32 + 4 * kq + r, n0 + wave * 32 + 16 * nb + i16, acc16[0][nb][r], acc16[NB - 1][nb][r]);
+    }
+    // 4x4 blocks: register r holds row r of the group, column lane % 32; the upper half of the wave
+    // holds the other float4 of every 8-k group
+#pragma unroll
+    for (int q = 0; q < G4; ++q)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = acc4[q][r] + __shfl_xor(acc4[q][r], 32);
+            if (kh == 0) emit(TAIL0 + 4 * q + r, n0 + wave * 32 + i32, v, 0.f);
+        }
+}
+
+// How `rows` rows are cut into 16-row units (two make a 32x32x2 block, an odd one a 16x16x4 block)
+// and 4-row groups: whole units, then one or two groups for a remainder of up to 8 rows when there
+// are at least two units to ride on; otherwise one more unit.  Measured on 32 uniform experts of
+// 128 + r rows: one group costs 44 % of a further unit, two 60 %, three 95 % (so three are not used);
+// on 4096 tokens over 32 experts (108..147 rows each) the layer gains 1.3 %.
+struct TileShape {
+    int nmb, g4;
+};
+template <bool GATED>
+__device__ __forceinline__ TileShape tile_shape(int rows) {
+    const int full = rows >> 4, rem = rows & 15;
+    if (GATED || rem == 0 || rem > 8 || full < 2) return TileShape{(rows + 15) >> 4, 0};
+    return TileShape{full, (rem + 3) >> 2};
+}
+
+template <int BN, bool GATED>
+__device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, float* C, int rows, const float* B0,
+                                              const float* B1, int n0, int N, int K, int epilogue, float* smem,
+                                              int a_alloc_rows) {
+    // the gated form keeps two accumulator sets, so its tiles are half as tall
+    constexpr int kMaxMb = (GATED ? kGemmTileRowsGated : kGemmTileRows) / 16;
+    // Tiles of up to 160 rows take K in steps of 64 floats (half as many barriers per flop); the LDS
+    // cannot hold two such stages of a taller tile or of two weight matrices, which take steps of 32.
+    const bool wide = !GATED && (K & 63) == 0;
+    const TileShape shape = tile_shape<GATED>(rows);
+#define INFMOE_CASE_G(n, g)                                                                                     \
+    case 4 * (n) + (g):                                                                                         \
+        if constexpr ((n) <= kMaxMb && ((g) == 0 || (!GATED && (n) >= 2 && (n) < kMaxMb))) {                    \
+            if constexpr (!GATED && 16 * (n) + 4 * (g) <= 16 * kMaxMb64) {                                      \
+                if (wide) {                                                                                     \
+                    gemm_tile<n, g, BN, GATED, 64>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem,             \
+                                                   min(a_alloc_rows, 16 * kMaxMb64));                           \
+                    break;                                                                                      \
+                }                                                                                               \
+            }                                                                                                   \
+            gemm_tile<n, g, BN, GATED, 32>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);      \
+        }                                                                                                       \
+        break;
+#define INFMOE_CASE(n) INFMOE_CASE_G(n, 0) INFMOE_CASE_G(n, 1) INFMOE_CASE_G(n, 2)
+    switch (4 * shape.nmb + shape.g4) {
+        INFMOE_CASE(1) INFMOE_CASE(2) INFMOE_CASE(3) INFMOE_CASE(4) INFMOE_CASE(5) INFMOE_CASE(6) INFMOE_CASE(7)
+        INFMOE_CASE(8) INFMOE_CASE(9) INFMOE_CASE(10) INFMOE_CASE(11) INFMOE_CASE(12) INFMOE_CASE(13)
+        INFMOE_CASE(14) INFMOE_CASE(15) INFMOE_CASE(16)
+        default: break;
+    }
+#undef INFMOE_CASE
+#undef INFMOE_CASE_G
+}
+
+// One expert: grid.x = column tiles, grid.y = row tiles of kGemmTileRows.
+template <int BN, bool GATED>
+__global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, int rows_total, int a_alloc_rows) {
+    extern __shared__ __align__(16) float smem[];
+    constexpr int kTile = GATED ? kGemmTileRowsGated : kGemmTileRows;
+    const int row0 = blockIdx.y * kTile;
+    const int rows = min(kTile, rows_total - row0);
+    const int n0 = blockIdx.x * BN;
+    gemm_dispatch<BN, GATED>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
+                             p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K, p.epilogue, smem,
+                             a_alloc_rows);
+}
+
+// All experts: 1-D grid of 8 * (row-tile capacity of an XCD) * n_col_tiles workgroups.  Workgroup id
+// b runs on XCD b % 8 and takes slot b / 8 of that XCD's share of the schedule: the share's row
+// tiles in descending height, all column tiles of a row tile in a row (they share its activations).
+template <int BN, bool GATED>
+__global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProblem p, size_t weight_stride,
+                                                                       const RowTile* __restrict__ tiles,
+                                                                       const int* __restrict__ sched,
+                                                                       int n_col_tiles) {
+    extern __shared__ __align__(16) float smem[];
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
+    if (slot >= share * n_col_tiles) return;
+    const RowTile rt = tiles[first + slot / n_col_tiles];
+    const int n0 = (slot % n_col_tiles) * BN;
+    const float* B0 = p.B + (size_t)rt.expert * weight_stride;
+    const float* B1 = GATED ? p.B1 + (size_t)rt.expert * weight_stride : nullptr;
+    gemm_dispatch<BN, GATED>(p.A + (size_t)rt.row0 * p.K, p.R ? p.R + (size_t)rt.row0 * p.N : nullptr,
+                             p.C + (size_t)rt.row0 * p.N, rt.rows, B0, B1, n0, p.N, p.K, p.epilogue, smem,
+                             GATED ? kGemmTileRowsGated : kGemmTileRows);
+}
+
+}  // namespace
+}  // namespace infmoe

@@ -23,6 +23,7 @@
 
 #include <type_traits>
 
+#include "device_math.h"
 #include "kernels.h"
 
 namespace infmoe {
@@ -33,12 +34,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
 constexpr int RW = 8;               // weight rows per wave
 constexpr int kWaves = kThreads / 64;
-
-__device__ __forceinline__ float gelu_dot(float a, float b) {
-    // plugin/cuda/ops/gelu.cu:8-15
-    const float cdf = 0.5f * (1.0f + tanhf(a * (0.035677408136300125f * a * a + 0.7978845608028654f)));
-    return a * cdf * b;
-}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -196,9 +196,12 @@ def run_t5ff(lib, torch, x, w, norm, ffn):
     return out.cpu().numpy()
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 5, 8, 9, 16, 17, 100, 128, 140, 255, 256, 257, 300, 600])
-def test_t5ff_row_counts(lib, torch_cuda, rows):
-    d, h = 64, 256
+# tile shapes (16-row units + 4-row groups): 33 -> 2+1, 40 -> 2+2, 44 -> 2+3, 45 -> 3+0, 49 -> 3+1 (an odd
+# unit and a group), 97 -> 6+1, 130 -> 8+1, 147 -> 9+1, 161 / 172 -> 10+1 / 10+3 (32-float steps), 250 -> 15+3
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 8, 9, 16, 17, 33, 40, 44, 45, 49, 97, 100, 128, 130, 140, 147, 161, 172,
+                                  250, 255, 256, 257, 300, 600])
+@pytest.mark.parametrize("d,h", [(64, 256), (256, 96)])  # 64-float and (h = 96) 32-float K steps
+def test_t5ff_row_counts(lib, torch_cuda, rows, d, h):
     w = O.draw_expert(21, 0, d, h, "relu")
     x = O.draw_inputs(rows, rows, d, 2)[0]
     got = run_t5ff(lib, torch_cuda, x, w, "rms", "relu")
