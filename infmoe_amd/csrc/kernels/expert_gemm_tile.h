@@ -304,11 +304,16 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
 struct TileShape {
     int nmb, g4;
 };
+// (Tiles of up to 160 rows carry groups only in their 64-float-step form, which K % 64 == 0 selects:
+// the 32-float-step form of those heights is instantiated without groups to keep the build short.)
 template <bool GATED>
-__device__ __forceinline__ TileShape tile_shape(int rows) {
+__device__ __forceinline__ TileShape tile_shape(int rows, bool wide) {
     const int full = rows >> 4, rem = rows & 15;
-    if (GATED || rem == 0 || rem > 8 || full < 2) return TileShape{(rows + 15) >> 4, 0};
-    return TileShape{full, (rem + 3) >> 2};
+    const TileShape units{(rows + 15) >> 4, 0};
+    if (GATED || rem == 0 || rem > 8 || full < 2) return units;
+    const TileShape groups{full, (rem + 3) >> 2};
+    if (!wide && 16 * groups.nmb + 4 * groups.g4 <= 16 * kMaxMb64) return units;
+    return groups;
 }
 
 template <int BN, bool GATED>
@@ -320,7 +325,7 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
     // Tiles of up to 160 rows take K in steps of 64 floats (half as many barriers per flop); the LDS
     // cannot hold two such stages of a taller tile or of two weight matrices, which take steps of 32.
     const bool wide = !GATED && (K & 63) == 0;
-    const TileShape shape = tile_shape<GATED>(rows);
+    const TileShape shape = tile_shape<GATED>(rows, wide);
 #define INFMOE_CASE_G(n, g)                                                                                     \
     case 4 * (n) + (g):                                                                                         \
         if constexpr ((n) <= kMaxMb && ((g) == 0 || (!GATED && (n) >= 2 && (n) < kMaxMb))) {                    \
@@ -331,7 +336,8 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
                     break;                                                                                      \
                 }                                                                                               \
             }                                                                                                   \
-            gemm_tile<n, g, BN, GATED, 32>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);      \
+            if constexpr ((g) == 0 || 16 * (n) + 4 * (g) > 16 * kMaxMb64)                                       \
+                gemm_tile<n, g, BN, GATED, 32>(A, R, C, rows, B0, B1, n0, N, K, epilogue, smem, a_alloc_rows);  \
         }                                                                                                       \
         break;
 #define INFMOE_CASE(n) INFMOE_CASE_G(n, 0) INFMOE_CASE_G(n, 1) INFMOE_CASE_G(n, 2)
