@@ -45,6 +45,8 @@ def run_gate(lib, torch, x, c, gamma, norm, bias=None, scratch=True):
     (16389, 256, 8, "rms", True),         # 64-token workgroups, ragged last group
     (40, 4096, 200, "rms", False),        # several passes over experts and several slices
     (1024, 1024, 32, "rms", False),       # 16-token workgroups, 4 slices
+    (40, 1030, 8, "rms", False),          # scalar path (row length not a multiple of 4) with slices
+    (7, 4098, 130, "none", False),        # scalar path, two passes over experts, slices
 ])
 @pytest.mark.parametrize("scratch", [True, False])
 def test_gate_top1_matches_oracle(lib, torch_cuda, T, d, E, norm, use_bias, scratch):
