@@ -258,26 +258,68 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     }
 
     // epilogue
+    // 32x32 block: register r holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    // 16x16 block: register r holds row 4*(lane/16) + r, column lane%16
+    // 4x4 blocks: register r holds row r of the group, column lane % 32; the upper half of the wave
+    // holds the other float4 of every 8-k group
+#pragma unroll
+    for (int q = 0; q < G4; ++q)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc4[q][r] += __shfl_xor(acc4[q][r], 32);
+    const bool residual = !GATED && epilogue == EPI_RESIDUAL;
+    if (residual) {
+        // The residual values of a block are fetched together before the first is used (from clamped,
+        // always valid addresses) and added to the accumulators: loaded next to its store inside the
+        // bounds check, every value would be waited for by itself, and the second GEMM of the
+        // sublayer then ran 3 % longer than the first.
+        const float* rcol = R + min(n0 + wave * 32 + i32, N - 1);
+        auto at = [&](const float* col, int row) { return col[(size_t)min(row, rows - 1) * N]; };
+#pragma unroll
+        for (int mb = 0; mb < N32; ++mb) {
+            float res[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) res[r] = at(rcol, 32 * mb + 8 * (r / 4) + 4 * kh + (r % 4));
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc32[0][mb][r] += res[r];
+        }
+        if (T16) {
+            float res[2][4];
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    res[nb][r] = at(R + min(n0 + wave * 32 + 16 * nb + i16, N - 1), 32 * N32 + 4 * kq + r);
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc16[0][nb][r] += res[nb][r];
+        }
+        if (G4 > 0) {
+            float res[G4 > 0 ? G4 : 1][4];
+#pragma unroll
+            for (int q = 0; q < G4; ++q)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) res[q][r] = at(rcol, TAIL0 + 4 * q + r);
+#pragma unroll
+            for (int q = 0; q < G4; ++q)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc4[q][r] += res[q][r];
+        }
+    }
     auto emit = [&](int row, int col, float v, float v1) {
         if (row < rows && col < N) {
-            const size_t o = (size_t)row * N + col;
-            if (GATED) {
+            if (GATED)
                 v = gelu_dot(v, v1);
-            } else if (epilogue == EPI_RELU) {
+            else if (!residual)
                 v = fmaxf(v, 0.f);
-            } else {
-                v += R[o];
-            }
-            C[o] = v;
+            C[(size_t)row * N + col] = v;
         }
     };
-    // 32x32 block: register r holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
 #pragma unroll
     for (int mb = 0; mb < N32; ++mb)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             emit(32 * mb + 8 * (r / 4) + 4 * kh + (r % 4), n0 + wave * 32 + i32, acc32[0][mb][r], acc32[NB - 1][mb][r]);
-    // 16x16 block: register r holds row 4*(lane/16) + r, column lane%16
     if (T16) {
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
@@ -285,15 +327,11 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             for (int r = 0; r < 4; ++r)
                 emit(32 * N32 + 4 * kq + r, n0 + wave * 32 + 16 * nb + i16, acc16[0][nb][r], acc16[NB - 1][nb][r]);
     }
-    // 4x4 blocks: register r holds row r of the group, column lane % 32; the upper half of the wave
-    // holds the other float4 of every 8-k group
 #pragma unroll
     for (int q = 0; q < G4; ++q)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float v = acc4[q][r] + __shfl_xor(acc4[q][r], 32);
-            if (kh == 0) emit(TAIL0 + 4 * q + r, n0 + wave * 32 + i32, v, 0.f);
-        }
+        for (int r = 0; r < 4; ++r)
+            if (kh == 0) emit(TAIL0 + 4 * q + r, n0 + wave * 32 + i32, acc4[q][r], 0.f);
 }
 
 // How `rows` rows are cut into 16-row units (two make a 32x32x2 block, an odd one a 16x16x4 block)
