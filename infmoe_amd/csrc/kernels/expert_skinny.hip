@@ -127,24 +127,26 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
         }
     }
 
+    // Lane m * RW + r stores output (row m, column n_base + r) and fetches its residual value before
+    // the reductions start (from a clamped, always valid address): loaded next to its store, each of
+    // the RW * M values would be waited for by itself.
+    static_assert(RW * M <= 64, "one lane per output");
+    const bool residual = !GATED && epilogue == EPI_RESIDUAL;
+    const int my_m = lane / RW, my_n = n_base + lane % RW;
+    float res = 0.f;
+    if (residual) res = R[(size_t)min(my_m, rows - 1) * N + min(my_n, N - 1)];
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
-        const int n = n_base + r;
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             float v = wave_sum(acc[0][r][m]);
-            float v1 = 0.f;
-            if (GATED) v1 = wave_sum(acc[NB - 1][r][m]);
-            if (lane == 0 && n < N && m < rows) {
-                const size_t o = (size_t)m * N + n;
-                if (GATED)
-                    v = gelu_dot(v, v1);
-                else if (epilogue == EPI_RELU)
-                    v = fmaxf(v, 0.f);
-                else
-                    v += R[o];
-                C[o] = v;
-            }
+            if (GATED)
+                v = gelu_dot(v, wave_sum(acc[NB - 1][r][m]));
+            else if (residual)
+                v += res;
+            else
+                v = fmaxf(v, 0.f);
+            if (lane == m * RW + r && my_n < N && m < rows) C[(size_t)m * N + my_n] = v;
         }
     }
     }  // row blocks
