@@ -66,30 +66,36 @@ def build_layer(torch, cfg, seed=0, keep_host=True, replicate=False):
     x = torch.randn(T, d, generator=gen, device="cuda")
     cent = (torch.randn(d, E, generator=gen, device="cuda") / d ** 0.5).t().contiguous()  # logical [d,E] -> [E][d]
     gamma = 1 + 0.1 * torch.randn(d, generator=gen, device="cuda")
+    gated = cfg.get("ffn", "relu") == "gated_gelu"
     mcfg = MoELayerConfig(seq_len=S, expert_count=E, embedding_size=d, hidden_size=h, max_concurrency=cfg["mc"],
                           moe_variant=cfg["variant"], sublayer_type="T5_FF", max_batch_size=B,
+                          ffn_kind=cfg.get("ffn", "relu"),
                           expert_centroids=cent.cpu().numpy(),
                           layernorm_weight=gamma.cpu().numpy() if cfg["variant"] == "cpm_2" else None)
     plugin = MoELayerPlugin(mcfg).create_plugin()
     slots = []
-    slot_floats = d + 2 * d * h
+    # [gamma | wi [h][d] | wo [d][h]], or [gamma | wi_0 | wi_1 | wo] for the gated form
+    inner = ("wi_0_weight", "wi_1_weight") if gated else ("wi_weight",)
+    slot_floats = d + (len(inner) + 1) * d * h
+
+    def hand_over(e, base):
+        plugin.set_expert_weights_ptr(e, "layer_norm_weight", base, d)
+        for i, name in enumerate(inner):
+            plugin.set_expert_weights_ptr(e, name, base + 4 * (d + i * d * h), d * h)
+        plugin.set_expert_weights_ptr(e, "wo_weight", base + 4 * (d + len(inner) * d * h), d * h)
+
     for e in range(E):
         if replicate and e > 0:  # profiling runs: every expert gets expert 0's values (same work, short set-up)
-            base = slots[0].ctypes.data if keep_host else slot.ctypes.data
-            plugin.set_expert_weights_ptr(e, "layer_norm_weight", base, d)
-            plugin.set_expert_weights_ptr(e, "wi_weight", base + 4 * d, d * h)
-            plugin.set_expert_weights_ptr(e, "wo_weight", base + 4 * (d + d * h), d * h)
+            hand_over(e, slots[0].ctypes.data if keep_host else slot.ctypes.data)
             if keep_host:
                 slots.append(slots[0])
             continue
-        slot = np.empty(slot_floats, np.float32)  # [gamma | wi [h][d] | wo [d][h]]
+        slot = np.empty(slot_floats, np.float32)
         slot[:d] = (1 + 0.1 * torch.randn(d, generator=gen, device="cuda")).cpu().numpy()
-        slot[d:d + d * h] = (torch.randn(h, d, generator=gen, device="cuda") / d ** 0.5).cpu().numpy().ravel()
-        slot[d + d * h:] = (torch.randn(d, h, generator=gen, device="cuda") / h ** 0.5).cpu().numpy().ravel()
-        base = slot.ctypes.data
-        plugin.set_expert_weights_ptr(e, "layer_norm_weight", base, d)
-        plugin.set_expert_weights_ptr(e, "wi_weight", base + 4 * d, d * h)
-        plugin.set_expert_weights_ptr(e, "wo_weight", base + 4 * (d + d * h), d * h)
+        for i in range(len(inner)):
+            slot[d + i * d * h:d + (i + 1) * d * h] = (torch.randn(h, d, generator=gen, device="cuda") / d ** 0.5).cpu().numpy().ravel()
+        slot[d + len(inner) * d * h:] = (torch.randn(d, h, generator=gen, device="cuda") / h ** 0.5).cpu().numpy().ravel()
+        hand_over(e, slot.ctypes.data)
         if keep_host:
             slots.append(slot)
     bias = None
@@ -130,6 +136,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-sample", type=int, default=4096)
+    ap.add_argument("--ffn", default="relu", choices=["relu", "gated_gelu"],
+                    help="relu: the two-matrix form the headline metric is quoted on; gated_gelu: the three-matrix "
+                         "form (an extra measurement, without the CPU leg)")
     ap.add_argument("--replicate-weights", action="store_true",
                     help="profiling aid: give every expert the values of expert 0 (short set-up, same work)")
     args = ap.parse_args()
@@ -143,7 +152,11 @@ def main():
     from infmoe_amd import capi
     capi.load()  # fails loudly when the HIP library has not been built
 
-    cfg = CONFIGS[args.config]
+    cfg = dict(CONFIGS[args.config], ffn=args.ffn)
+    gated = args.ffn == "gated_gelu"
+    if gated:
+        args.no_cpu = True
+    n_mat = 3 if gated else 2  # weight matrices of an expert
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = cfg["shape"]
     T = B * S
@@ -181,10 +194,14 @@ def main():
 
     resident = cfg["mc"] >= E
     few_rows = T <= 16 * E  # same rule the sub-layer uses to pick the few-row kernels
-    gemm_ms = 0.5 * (phases["expert_gemm1"] + phases["expert_gemm2"])
+    # average launch of the two expert kernels; the gated form's first launch takes two matrices, so its
+    # figures are per matrix: (time of both launches) / 3
+    gemm_ms = (phases["expert_gemm1"] + phases["expert_gemm2"]) / n_mat
+    launches = ("two launches per step: wi_0 and wi_1 with gelu*mul, wo with residual; figures per weight matrix"
+                if gated else "two launches per step: wi with ReLU, wo with residual")
     if not resident:
         # streamed experts: the host link bounds the call; report the achieved copy rate
-        bytes_per_call = active * 4.0 * (d + 2 * d * h)
+        bytes_per_call = active * 4.0 * (d + n_mat * d * h)
         roofline = {"bound": "hbm", "achieved": round(bytes_per_call / (phases["expert_gemm1"] * 1e-3) / 1e9, 2),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": None,
                     "kernel": "host-to-device expert copies overlapped with expert kernels",
@@ -192,15 +209,16 @@ def main():
     elif few_rows:
         bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
         roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                    "kernel": "expert_skinny_kernel (two launches per step: wi with ReLU, wo with residual)",
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "traffic": None if gated else MEASURED_TRAFFIC_BYTES.get(args.config),
+                    "kernel": f"expert_skinny_kernel ({launches})",
                     "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     else:
         flops_per_launch = 2.0 * T * d * h
         roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
                     "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                    "kernel": "expert_gemm_grouped_kernel (two launches per step: wi with ReLU, wo with residual)",
+                    "traffic": None if gated else MEASURED_TRAFFIC_BYTES.get(args.config),
+                    "kernel": f"expert_gemm_grouped_kernel ({launches})",
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
 
@@ -219,7 +237,7 @@ def main():
         "data": "synthetic" + (" (expert 0 replicated)" if args.replicate_weights else ""),
         "config": {"workload": f"{args.config}: {cfg['variant']} E={E} d={d} h={h} tokens={T} ({B}x{S}) "
                                f"max_concurrency={cfg['mc']} ({'resident' if resident else 'streamed'} experts), "
-                               f"T5_FF rms norm + relu", "tokens": T, "active_experts": active,
+                               f"T5_FF rms norm + {'gated gelu (three matrices)' if gated else 'relu'}", "tokens": T, "active_experts": active,
                    "tokens_per_expert_min_max": [int(count.min()), int(count.max())]},
         "roofline": roofline,
         "phases_ms": {k: round(v, 4) for k, v in phases.items()},

@@ -81,7 +81,7 @@ __device__ __forceinline__ void scan_body(int T, int E, int nblk, int* __restric
             const int c = s_count[e];
             s_off[e] = off;
             s_tile0[e] = nt;
-            if (c > skinny_max) nt += (c + tile_rows - 1) / tile_rows;
+            if (c > skinny_max) nt += (c + tile_rows - 1) / tile_rows;  // tiles of row_tile_height(c, tile_rows)
             off += c;
         }
         s_total = off;
@@ -97,11 +97,12 @@ __device__ __forceinline__ void scan_body(int T, int E, int nblk, int* __restric
         const int c = s_count[e];
         if (c <= skinny_max) continue;
         int j = s_tile0[e];
-        for (int m0 = 0; m0 < c; m0 += tile_rows, ++j) {
+        const int per = row_tile_height(c, tile_rows);
+        for (int m0 = 0; m0 < c; m0 += per, ++j) {
             RowTile rt;
             rt.expert = e;
             rt.row0 = s_off[e] + m0;
-            rt.rows = min(tile_rows, c - m0);
+            rt.rows = min(per, c - m0);
             rt.pad = 0;
             if (sorted)
                 s_raw[j] = rt;

@@ -69,20 +69,21 @@ hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t wei
     return hipGetLastError();
 }
 
-hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream) {
+hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
+    if (tile_rows <= 0 || tile_rows % 16 != 0 || tile_rows > gemm_tile_rows(p.epilogue)) return hipErrorInvalidValue;
     if (!fast_path_ok(p)) {
         const size_t n = (size_t)rows * p.N;
         expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows, 0, nullptr);
         return hipGetLastError();
     }
-    const int tile = gemm_tile_rows(p.epilogue);
-    const int a_alloc = std::min(tile, ((rows + 31) / 32) * 32);  // whole 32-row slabs
+    const int tile = std::min(row_tile_height(rows, tile_rows), ((rows + 15) / 16) * 16);
+    const int a_alloc = ((tile + 31) / 32) * 32;  // whole 32-row slabs
     const dim3 grid((p.N + kGemmColumns - 1) / kGemmColumns, (rows + tile - 1) / tile);
     const bool gated = p.epilogue == EPI_GATED_GELU;
     const size_t lds = lds_bytes(gated, a_alloc, p.K);
-    return gated ? expert_gemm_launch_one_gated(p, rows, a_alloc, grid, lds, stream)
-                 : expert_gemm_launch_one(p, rows, a_alloc, grid, lds, stream);
+    return gated ? expert_gemm_launch_one_gated(p, rows, tile, a_alloc, grid, lds, stream)
+                 : expert_gemm_launch_one(p, rows, tile, a_alloc, grid, lds, stream);
 }
 
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,

@@ -4,11 +4,11 @@
 
 namespace infmoe {
 
-hipError_t expert_gemm_launch_one(const GemmProblem& p, int rows, int a_alloc_rows, dim3 grid, size_t lds,
-                                  hipStream_t stream) {
+hipError_t expert_gemm_launch_one(const GemmProblem& p, int rows, int tile_rows, int a_alloc_rows, dim3 grid,
+                                  size_t lds, hipStream_t stream) {
     const hipError_t err = allow_lds_once<expert_gemm_kernel<kGemmColumns, false>>(kLdsPerCu);
     if (err != hipSuccess) return err;
-    expert_gemm_kernel<kGemmColumns, false><<<grid, kGemmThreads, lds, stream>>>(p, rows, a_alloc_rows);
+    expert_gemm_kernel<kGemmColumns, false><<<grid, kGemmThreads, lds, stream>>>(p, rows, tile_rows, a_alloc_rows);
     return hipGetLastError();
 }
 

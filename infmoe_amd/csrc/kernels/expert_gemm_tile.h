@@ -389,13 +389,13 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
 #undef INFMOE_CASE_G
 }
 
-// One expert: grid.x = column tiles, grid.y = row tiles of kGemmTileRows.
+// One expert: grid.x = column tiles, grid.y = row tiles of tile_rows rows (the last may be shorter).
 template <int BN, bool GATED>
-__global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, int rows_total, int a_alloc_rows) {
+__global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, int rows_total, int tile_rows,
+                                                               int a_alloc_rows) {
     extern __shared__ __align__(16) float smem[];
-    constexpr int kTile = GATED ? kGemmTileRowsGated : kGemmTileRows;
-    const int row0 = blockIdx.y * kTile;
-    const int rows = min(kTile, rows_total - row0);
+    const int row0 = blockIdx.y * tile_rows;
+    const int rows = min(tile_rows, rows_total - row0);
     const int n0 = blockIdx.x * BN;
     gemm_dispatch<BN, GATED>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
                              p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K, p.epilogue, smem,

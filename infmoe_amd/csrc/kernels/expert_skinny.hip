@@ -154,7 +154,7 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
 
 // count == nullptr: one expert with `rows_fixed` rows at row 0; else blockIdx.y is the expert.
 template <bool GATED>
-__global__ __launch_bounds__(kThreads, 3) void expert_skinny_kernel(GemmProblem p, size_t weight_stride,
+__global__ __launch_bounds__(kThreads, GATED ? 2 : 3) void expert_skinny_kernel(GemmProblem p, size_t weight_stride,
                                                                  const int* __restrict__ count,
                                                                  const int* __restrict__ offset, int rows_fixed,
                                                                  int row_blocks) {

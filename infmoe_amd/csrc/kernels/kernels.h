@@ -45,6 +45,18 @@ size_t expert_count_scratch_bytes(int T, int E);
 constexpr int kXcdCount = 8;    // accelerator dies of an MI355X; workgroup ids are dealt to them round-robin
 constexpr int kSchedInts = 16;  // [0] number of row tiles, [1..9] first tile of each XCD's share
 inline int max_row_tiles(int T, int E, int tile_rows) { return (T + tile_rows - 1) / tile_rows + E; }
+// Height of the row tiles an expert's `rows` rows are cut into when no tile may exceed `tile_rows` (a
+// multiple of 16): as few tiles as that allows, all of one height (a multiple of 16; the last tile
+// takes what is left), so that 300 rows become 160 + 140 rather than 256 + 44.  The grouped and the
+// one-expert launches both cut by this rule: which matrix instruction a row meets depends on its
+// place in its tile, and the two schedules have to agree bit for bit.
+#if defined(__HIPCC__)
+__host__ __device__
+#endif
+inline int row_tile_height(int rows, int tile_rows) {
+    const int n = (rows + tile_rows - 1) / tile_rows;
+    return n <= 1 ? tile_rows : ((rows + n - 1) / n + 15) / 16 * 16;
+}
 // Most row tiles one XCD may be given (bounds the grid of the grouped launch).
 inline int xcd_tile_capacity(int max_tiles) {
     const int cap = 2 * ((max_tiles + kXcdCount - 1) / kXcdCount) + 8;
@@ -90,8 +102,10 @@ struct GemmProblem {
     int N, K;
     int epilogue;
 };
-// One expert, `rows` known on the host.
-hipError_t launch_expert_gemm(const GemmProblem& p, int rows, hipStream_t stream);
+// One expert, `rows` known on the host, cut into row tiles of at most `tile_rows` rows (a multiple of
+// 16 no larger than gemm_tile_rows(p.epilogue); both launches of a sub-layer pass the same value so
+// that they cut the rows as the grouped launch does).
+hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hipStream_t stream);
 // All experts in one launch: A, R, C address routed rows globally; expert e's weights are at
 // B + e*weight_stride (floats).  Row tiles and their number come from launch_expert_count.
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
@@ -103,7 +117,7 @@ bool expert_gemm_grouped_ok(const GemmProblem& p, size_t weight_stride);
 hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t weight_stride, const int* row_expert,
                                                 int rows, hipStream_t stream);
 constexpr int kGemmTileRows = 256;       // tallest row tile of the GEMM kernel
-constexpr int kGemmTileRowsGated = 128;  // ... of its two-matrix (gated) form
+constexpr int kGemmTileRowsGated = 192;  // ... of its two-matrix (gated) form (two accumulator sets)
 inline int gemm_tile_rows(int epilogue) { return epilogue == EPI_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
 
 // Few-row experts (decode): every weight row is streamed once and dotted with up to

@@ -171,8 +171,10 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
         INFMOE_HIP(launch_expert_skinny(g1, rows, stream));
         INFMOE_HIP(launch_expert_skinny(g2, rows, stream));
     } else {
-        INFMOE_HIP(launch_expert_gemm(g1, rows, stream));
-        INFMOE_HIP(launch_expert_gemm(g2, rows, stream));
+        // both launches cut the rows as the grouped schedule does (rowTileHeight())
+        const int tileRows = ffnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows;
+        INFMOE_HIP(launch_expert_gemm(g1, rows, tileRows, stream));
+        INFMOE_HIP(launch_expert_gemm(g2, rows, tileRows, stream));
     }
     return INFMOE_OK;
 }

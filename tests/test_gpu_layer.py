@@ -147,16 +147,20 @@ def test_decode_shape_uses_few_row_kernels_and_matches(torch_cuda):
         plugin.terminate()
 
 
-def test_skewed_routing_with_score_bias(torch_cuda):
+@pytest.mark.parametrize("ffn", ["relu", "gated_gelu"])
+def test_skewed_routing_with_score_bias(torch_cuda, ffn):
+    """Experts of very different sizes, some cut into several row tiles (of equal height): the grouped
+    and the per-expert launches cut alike, so both schedules give the same bits."""
     shape, E, d, h = (8, 256), 16, 128, 256
     x, c, _ = O.draw_inputs(17, 8 * 256, d, E)
     bias = O.zipf_score_bias(x, c, s=1.2)
     outs = []
     for mc in (E, 3):  # resident; streamed, where the experts run largest first
-        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "base_layer", seed=17, bias=bias)
-        y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "base_layer", bias=bias)
+        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "base_layer", ffn=ffn, seed=17, bias=bias)
+        y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "base_layer", ffn=ffn, bias=bias)
         assert count.max() > 4 * max(count.min(), 1)  # the histogram really is skewed
         assert count.max() > 256                      # and some expert needs more than one row tile
+        assert ((count > 128) & (count <= 256)).any()  # and one lies between the tile heights of the two forms
         outs.append(y)
         plugin.terminate()
     np.testing.assert_array_equal(outs[0], outs[1])
