@@ -35,10 +35,23 @@ constexpr int kThreads = 256;
 constexpr int RW = 8;               // weight rows per wave
 constexpr int kWaves = kThreads / 64;
 
+// v + (v of the lane that the data-parallel-primitive control CTRL names): a register-to-register move
+// inside a row of 16 lanes, no trip through the LDS crossbar as a shuffle by lane index takes
+template <int CTRL>
+__device__ __forceinline__ float add_dpp(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// Sum over the wave, the same value in every lane: four steps inside the rows of 16 lanes (lane ^ 1,
+// lane ^ 2, mirror in 8, mirror in 16), then the four row sums read as scalars.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v = add_dpp<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+    v = add_dpp<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+    v = add_dpp<0x141>(v);  // row_half_mirror
+    v = add_dpp<0x140>(v);  // row_mirror
+    const int bits = __float_as_int(v);
+    const float s0 = __int_as_float(__builtin_amdgcn_readlane(bits, 0)), s1 = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    const float s2 = __int_as_float(__builtin_amdgcn_readlane(bits, 32)), s3 = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+    return (s0 + s1) + (s2 + s3);
 }
 
 // SEG: 16-byte loads per lane per weight row per chunk; RPN: weight rows loaded together
