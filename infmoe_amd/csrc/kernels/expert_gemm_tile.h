@@ -1,6 +1,6 @@
 // FP32 matrix-core GEMM of the T5 feed-forward expert for gfx950: device code.
 // Included by the translation units that instantiate one kernel each (the tile body exists in some
-// seventy shapes per kernel, so they compile side by side).
+// sixty shapes per one-matrix kernel, so they compile side by side).
 //
 // Replaces the three cublasSgemm_v2 calls, the thrust gelu*mul pass and the device-to-device
 // residual copy of T5FFLayer::run (plugin/sublayers/T5FFLayer.cc:112-138, plugin/cuda/ops/gelu.cu:7-25):
@@ -13,20 +13,21 @@
 // block at the bottom of a tile so that row counts are padded to 16, not 32.
 //
 // Tiling.  The weights are the big operand (335 MB per expert at d=4096, h=10240) and each weight
-// element is reused only `rows` times, so a workgroup covers ALL rows of its expert (up to 256) x
-// BN weight rows: every weight byte is fetched from HBM once.  Token counts per expert vary, so the
+// element is reused only `rows` times, so a workgroup covers ALL rows of its expert (up to 256, or
+// 192 with two weight matrices; a taller expert is cut into equal tiles, see row_tile_height) x BN
+// weight rows: every weight byte is fetched from HBM once.  Token counts per expert vary, so the
 // tile height is a run-time multiple of 16 rows (NMB of them: NMB/2 blocks of 32 rows plus one of
-// 16 when NMB is odd); the body is instantiated for NMB = 1..16 and selected per workgroup, which
-// wastes at most 15 padded rows per expert instead of up to a whole fixed-height tile.  The 4
-// waves of a workgroup split the BN = 128 columns, 32 each, and keep the accumulators of all row
-// blocks in registers.
+// 16 when NMB is odd) plus up to two groups of 4 rows; the body is instantiated for NMB = 1..16 and
+// selected per workgroup, which wastes at most 3 padded rows per expert (15 where the groups are
+// not used) instead of up to a whole fixed-height tile.  The 4 waves of a workgroup split the
+// BN = 128 columns, 32 each, and keep the accumulators of all row blocks in registers.
 //
-// Pipeline.  K advances in steps of 32 floats.  While the matrix core works on step s from one half
+// Pipeline.  K advances in steps of BK = 32 or 64 floats.  While the matrix core works on step s from one half
 // of a double-buffered LDS tile, the global loads of step s+2 go into registers and the registers
 // holding step s+1 are written to the other half; one barrier per step.  These memory operations
 // are not issued in bursts before and after the MFMAs (that left the matrix core idle a quarter of
-// the time) but dealt out a few at a time between small groups of MFMAs.  LDS rows are padded to 36 floats so that the 16-byte
-// operand reads of the lanes of a block hit distinct banks.  Inside an 8-float (32x32x2) or 16-float
+// the time) but dealt out a few at a time between small groups of MFMAs.  LDS rows are padded to
+// BK + 4 floats so that the 16-byte operand reads of the lanes of a block hit distinct banks.  Inside an 8-float (32x32x2) or 16-float
 // (16x16x4) chunk the k order is permuted identically for A and B (lane group q supplies floats
 // 4q..4q+3 over four instructions), which a dot product does not see and which lets every operand
 // read be a ds_read_b128.
