@@ -210,6 +210,16 @@ def test_t5ff_row_counts(lib, torch_cuda, rows, d, h):
     assert_close(got, O.t5ff_run(x, w, "rms", "relu"), what=f"t5ff rows={rows}")
 
 
+# the two-matrix form keeps two accumulator sets: tiles of up to 192 rows, taller experts in equal tiles
+@pytest.mark.parametrize("rows", [9, 130, 192, 193, 400])
+def test_t5ff_gated_row_counts(lib, torch_cuda, rows):
+    d, h = 64, 256
+    w = O.draw_expert(24, 0, d, h, "gated_gelu")
+    x = O.draw_inputs(rows, rows, d, 2)[0]
+    got = run_t5ff(lib, torch_cuda, x, w, "centered", "gated_gelu")
+    assert_close(got, O.t5ff_run(x, w, "centered", "gated_gelu"), what=f"gated t5ff rows={rows}")
+
+
 @pytest.mark.parametrize("d,h", [(64, 256), (128, 320), (20, 36), (6, 10), (512, 1280), (4096, 256)])
 @pytest.mark.parametrize("norm,ffn", [("rms", "relu"), ("centered", "gated_gelu"), ("rms", "gated_gelu"), ("centered", "relu")])
 @pytest.mark.parametrize("rows", [4, 70])
