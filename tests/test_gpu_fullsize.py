@@ -80,6 +80,20 @@ def test_full_size_layer_sampled_rows(lib, torch_cuda, name, experts_to_check, r
     plugin.terminate()
 
 
+def test_full_size_streamed_equals_resident(torch_cuda):
+    """The same layer with its experts streamed through two slots (10.7 GB over the host link per call)
+    and with all of them resident: the same bits."""
+    torch = torch_cuda
+    import bench
+    outs = []
+    for name in ("c2", "c3"):  # equal but for max_concurrency: 32 (resident) and 2
+        plugin, x, *_ = bench.build_layer(torch, bench.CONFIGS[name], keep_host=False)
+        outs.append(plugin.forward(x.contiguous()).clone())
+        torch.cuda.synchronize()
+        plugin.terminate()
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_full_size_identity_returns_input(torch_cuda):
     torch = torch_cuda
     T, d, E = 4096, 4096, 32
