@@ -15,7 +15,10 @@ from tests.gpu_util import assert_close, check_assignment, stream_ptr
 pytestmark = pytest.mark.gpu
 
 
-def slot_weights(slot, d, h):
+def slot_weights(slot, d, h, ffn):
+    if ffn == "gated_gelu":
+        return {"layer_norm_weight": slot[:d], "wi_0_weight": slot[d:d + d * h].reshape(h, d),
+                "wi_1_weight": slot[d + d * h:d + 2 * d * h].reshape(h, d), "wo_weight": slot[d + 2 * d * h:].reshape(d, h)}
     return {"layer_norm_weight": slot[:d], "wi_weight": slot[d:d + d * h].reshape(h, d),
             "wo_weight": slot[d + d * h:].reshape(d, h)}
 
@@ -35,11 +38,13 @@ def device_gate(lib, torch, x2d, cent, gamma, norm, bias):
     return sel.cpu().numpy(), coeff.cpu().numpy(), stats.cpu().numpy()
 
 
-@pytest.mark.parametrize("name,experts_to_check,rows_per_expert", [("c2", 2, 24), ("c5", 5, 8), ("c4", 3, 16)])
-def test_full_size_layer_sampled_rows(lib, torch_cuda, name, experts_to_check, rows_per_expert):
+# the last case is the three-matrix form the reference's code computes, at c2's sizes
+@pytest.mark.parametrize("name,experts_to_check,rows_per_expert,ffn",
+                         [("c2", 2, 24, "relu"), ("c5", 5, 8, "relu"), ("c4", 3, 16, "relu"), ("c2", 2, 16, "gated_gelu")])
+def test_full_size_layer_sampled_rows(lib, torch_cuda, name, experts_to_check, rows_per_expert, ffn):
     torch = torch_cuda
     import bench
-    cfg = bench.CONFIGS[name]
+    cfg = dict(bench.CONFIGS[name], ffn=ffn)
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = cfg["shape"]
     T = B * S
@@ -68,9 +73,9 @@ def test_full_size_layer_sampled_rows(lib, torch_cuda, name, experts_to_check, r
     chosen = list(dict.fromkeys([order[0], order[-1], *order[:: max(1, len(order) // experts_to_check)]]))[:experts_to_check]
     checked = 0
     for e in chosen:
-        w = slot_weights(slots[e], d, h)
+        w = slot_weights(slots[e], d, h, ffn)
         toks = np.flatnonzero(sel == e)[:rows_per_expert]
-        post = O.t5ff_run(xh[toks], w, "rms", "relu")
+        post = O.t5ff_run(xh[toks], w, "rms", ffn)
         if variant == "base_layer":
             a = O.sigmoid(aff[toks, e])[:, None]
             post = a * post + (1 - a) * xh[toks].astype(np.float64)
