@@ -222,6 +222,20 @@ def main():
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
 
+    # the bandwidth-bound phases: algorithmic bytes / phase time (the phase times include the launch
+    # gaps and the event marks, a few microseconds each), against the HBM peak
+    cpm2 = cfg["variant"] == "cpm_2"
+    mix = cfg["variant"] == "base_layer"
+    phase_bytes = {
+        "gating": 4.0 * (T * d + E * d + (d if cpm2 else 0) + 2 * T),
+        "scatter": 4.0 * (2 * T * d + T + (2 * T if mix else 0)),
+        "expert_norm": 4.0 * (2 * T * d + d),
+        "gather": 4.0 * ((3 * T * d + 2 * T) if mix else (2 * T * d + T)),
+    }
+    phase_rates = {k: {"bytes": v, "GB/s": round(v / (phases[k] * 1e-3) / 1e9, 1),
+                       "frac_of_hbm_peak": round(v / (phases[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                   for k, v in phase_bytes.items() if phases.get(k, 0) > 0}
+
     out = {
         "metric": f"MoE-layer tokens/s (E={E},d={d},h={h},fp32)",
         "value": round(T / (ms_per_step * 1e-3), 1),
@@ -242,6 +256,7 @@ def main():
         "roofline": roofline,
         "phases_ms": {k: round(v, 4) for k, v in phases.items()},
         "phases_ms_last_timed_step": {k: round(v, 4) for k, v in last.items()},
+        "phase_rates": phase_rates,
         "host_ms_per_step": round(wall_ms, 4),
         "routing": stats,
     }
