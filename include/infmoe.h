@@ -196,6 +196,22 @@ size_t infmoe_expert_count_scratch_bytes(int32_t T, int32_t E);
 int32_t infmoe_expert_count(int32_t T, int32_t E, const int32_t* sel, int32_t* pos, int32_t* count, int32_t* offset,
                             void* scratch, void* hip_stream);
 
+/*
+ * The same computation as infmoe_expert_count for callers that cannot allocate device memory
+ * and have no scratch to pass (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  The block-histogram scratch lives
+ * in a device array inside the library, INFMOE_EXPERT_COUNT_NOALLOC_MAX_INTS int32 (256 KiB)
+ * on every GPU the library runs on, held until the process ends.  The call allocates nothing
+ * (no hipMalloc / hipFree, on the first call neither) and returns INFMOE_ERR_INVALID_ARGUMENT
+ * when ceil(T / 1024) * E (rounded up to 64) exceeds that many ints.  All calls on one GPU share
+ * the array: calls that overlap there (different streams, different threads) race; calls on one
+ * stream are ordered.  Nothing has to be cleared between calls.  The first call on a device
+ * looks up the array's address and must not be made while a stream capture is in progress.
+ */
+#define INFMOE_EXPERT_COUNT_NOALLOC_MAX_INTS 65536
+int32_t infmoe_expert_count_noalloc(int32_t T, int32_t E, const int32_t* sel, int32_t* pos, int32_t* count,
+                                    int32_t* offset, void* hip_stream);
+
 /* Replaces moe_expert_scatter (plugin/cuda/moe.cu:214-228): routed[r,:] = x[pos[r],:],
  * routed_coeff[r] = coeff[pos[r]] (coeff / routed_coeff may both be NULL). */
 int32_t infmoe_expert_scatter(int32_t T, int32_t d, const float* x, const float* coeff, const int32_t* pos,

@@ -60,6 +60,7 @@ PROTOTYPES = {
     "infmoe_gate_top1": (_i32, [_i32, _i32, _i32, _pf, _pf, _pf, _i32, _pf, _vp, _pf, _vp, _vp, _vp]),
     "infmoe_expert_count_scratch_bytes": (_sz, [_i32, _i32]),
     "infmoe_expert_count": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "infmoe_expert_count_noalloc": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "infmoe_expert_scatter": (_i32, [_i32, _i32, _pf, _pf, _vp, _pf, _pf, _vp]),
     "infmoe_expert_gather": (_i32, [_i32, _i32, _pf, _vp, _pf, _vp]),
     "infmoe_expert_mix_gather": (_i32, [_i32, _i32, _vp, _pf, _pf, _pf, _pf, _vp]),

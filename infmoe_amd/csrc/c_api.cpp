@@ -245,6 +245,8 @@ const char* infmoe_plugin_version(void) { return "1"; }
 #define INFMOE_NEED(cond, msg) \
     if (!(cond)) return fail(INFMOE_ERR_INVALID_ARGUMENT, msg)
 
+static_assert(kExpertCountStaticInts == INFMOE_EXPERT_COUNT_NOALLOC_MAX_INTS, "header and kernel disagree on the limit");
+
 size_t infmoe_gate_top1_scratch_bytes(int32_t T, int32_t d, int32_t E) {
     return sizeof(float) * gate_scratch_floats(T < 0 ? 0 : T, d < 1 ? 1 : d, E < 1 ? 1 : E);
 }
@@ -276,6 +278,22 @@ int32_t infmoe_expert_count(int32_t T, int32_t E, const int32_t* sel, int32_t* p
         INFMOE_NEED(count && offset && (T == 0 || (sel && pos && scratch)), "expert_count: null pointer");
         INFMOE_HIP(launch_expert_count(T, E, sel, pos, count, offset, scratch, nullptr, nullptr, kGemmTileRows, 0,
                                        nullptr, static_cast<hipStream_t>(hip_stream)));
+        return INFMOE_OK;
+    });
+}
+
+int32_t infmoe_expert_count_noalloc(int32_t T, int32_t E, const int32_t* sel, int32_t* pos, int32_t* count,
+                                    int32_t* offset, void* hip_stream) {
+    return guarded([&]() -> int32_t {
+        INFMOE_NEED(T >= 0 && E > 0, "expert_count_noalloc: bad sizes");
+        INFMOE_NEED(count && offset && (T == 0 || (sel && pos)), "expert_count_noalloc: null pointer");
+        const size_t need = expert_count_scratch_bytes(T, E) / sizeof(int32_t);
+        if (need > (size_t)INFMOE_EXPERT_COUNT_NOALLOC_MAX_INTS)
+            return fail(INFMOE_ERR_INVALID_ARGUMENT,
+                        "expert_count_noalloc: ceil(T/1024)*E = %zu ints of scratch exceed the built-in %d; use "
+                        "infmoe_expert_count with caller-supplied scratch",
+                        need, INFMOE_EXPERT_COUNT_NOALLOC_MAX_INTS);
+        INFMOE_HIP(launch_expert_count_static(T, E, sel, pos, count, offset, static_cast<hipStream_t>(hip_stream)));
         return INFMOE_OK;
     });
 }

@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 
 #include <initializer_list>
+#include <mutex>
 
 #include "device_math.h"
 #include "kernels.h"
@@ -356,6 +357,47 @@ hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* coun
                                             xcd_tile_capacity(max_tiles), tile_rows, skinny_max);
     if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);
     return hipGetLastError();
+}
+
+// ---- the same three kernels with their block-histogram scratch in a device array of the library
+// instead of in memory the caller brings.  The array exists once per GPU (each device holds its own
+// copy at its own address); its address is looked up once per device, with that device current, and
+// kept.  Host code never passes the array's name to a kernel: the name is a host-side handle of the
+// symbol, not a device address.
+namespace {
+static __device__ __align__(256) int g_count_scratch[kExpertCountStaticInts];
+constexpr int kMaxDevices = 64;
+
+hipError_t static_count_scratch(int** out) {
+    static std::mutex lock;
+    static int* ptrs[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (ptrs[dev] == nullptr) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(g_count_scratch));
+        if (err != hipSuccess) return err;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        ptrs[dev] = static_cast<int*>(p);
+    }
+    *out = ptrs[dev];
+    return hipSuccess;
+}
+}  // namespace
+
+hipError_t launch_expert_count_static(int T, int E, const int* sel, int* pos, int* count, int* offset,
+                                      hipStream_t stream) {
+    if (expert_count_scratch_bytes(T, E) > sizeof(int) * kExpertCountStaticInts) return hipErrorInvalidValue;
+    int* blockhist = nullptr;
+    const hipError_t err = static_count_scratch(&blockhist);
+    if (err != hipSuccess) return err;
+    // every entry the scan and the ranking read is written by the histogram of the same call, so
+    // nothing of an earlier call's contents has to be cleared
+    return launch_expert_count(T, E, sel, pos, count, offset, blockhist, nullptr, nullptr, kGemmTileRows, 0, nullptr,
+                               stream);
 }
 
 hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream) {

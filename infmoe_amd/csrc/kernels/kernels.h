@@ -71,6 +71,13 @@ hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* coun
                                RowTile* tiles, int* sched, int tile_rows, int skinny_max, int* row_expert,
                                hipStream_t stream);
 
+// The same with the scratch in a device array owned by the library (kExpertCountStaticInts ints per GPU,
+// held until the process ends): no allocation and no caller-supplied scratch.  Calls on one GPU share
+// the array, so calls that overlap there race.  hipErrorInvalidValue when the scratch would not fit.
+constexpr size_t kExpertCountStaticInts = 64 * 1024;
+hipError_t launch_expert_count_static(int T, int E, const int* sel, int* pos, int* count, int* offset,
+                                      hipStream_t stream);
+
 // Small fill kernel (used instead of hipMemsetAsync so that callers may capture the layer in a graph).
 hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream);
 
