@@ -159,6 +159,15 @@ int32_t infmoe_serialization_size(const infmoe_plugin* p, size_t* out_bytes);
 int32_t infmoe_serialize(const infmoe_plugin* p, void* buffer, size_t buffer_bytes);
 int32_t infmoe_deserialize(const char* layer_name, const void* data, size_t bytes, infmoe_plugin** out);
 
+/*
+ * Replaces cnpy::npz_load for one array (plugin/thirdparty/cnpy/cnpy.cpp:229-276, used at
+ * plugin/sublayers/T5FFLayer.cc:143-147): reads float32 member `name` (e.g. "3/wo_weight",
+ * README.md:121) of the .npz archive `path` into `dst_host` in C order.  The member must be
+ * little-endian float32 of shape (rows, cols), or (rows,) when cols == 0; stored and deflated
+ * members, zip64 archives and Fortran-ordered 2-D members are read.  Host memory only: needs no GPU.
+ */
+int32_t infmoe_npz_read_f32(const char* path, const char* name, float* dst_host, size_t rows, size_t cols);
+
 const char* infmoe_last_error(void);
 const char* infmoe_plugin_name(void);    /* "MoELayerPlugin", plugin/MoELayerPlugin.h:18-19 */
 const char* infmoe_plugin_version(void); /* "1" */

@@ -1,6 +1,7 @@
 """Build libinfmoe.so (host C++ + gfx950 HIP kernels) in-tree with hipcc.
 
-    python -m infmoe_amd.build            # compile every source, then link
+    python -m infmoe_amd.build                 # compile every source, then link
+    python -m infmoe_amd.build --incremental   # recompile only what is older than its source or any header
 Objects go to infmoe_amd/csrc/build/, the library to infmoe_amd/lib/libinfmoe.so.
 """
 from __future__ import annotations
@@ -39,8 +40,20 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result"]
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def _compile(src: str) -> str:
+def _newest_header() -> float:
+    newest = os.path.getmtime(os.path.join(HERE, "..", "include", "infmoe.h"))
+    for root, _, files in os.walk(CSRC):
+        for f in files:
+            if f.endswith(".h"):
+                newest = max(newest, os.path.getmtime(os.path.join(root, f)))
+    return newest
+
+
+def _compile(src: str, incremental: bool = False) -> str:
     obj = os.path.join(OBJ_DIR, src.replace("/", "_") + ".o")
+    if incremental and os.path.isfile(obj):
+        if os.path.getmtime(obj) > max(os.path.getmtime(os.path.join(CSRC, src)), _newest_header()):
+            return obj
     cmd = [HIPCC, *COMMON, *DEVICE, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -51,11 +64,11 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(jobs: int = 8) -> str:
+def build(jobs: int = 8, incremental: bool = False) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(_compile, SOURCES))
+        objs = list(pool.map(lambda s: _compile(s, incremental), SOURCES))
     cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-lz", "-o", LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -64,4 +77,4 @@ def build(jobs: int = 8) -> str:
 
 
 if __name__ == "__main__":
-    print(build())
+    print(build(incremental="--incremental" in sys.argv[1:]))

@@ -53,6 +53,7 @@ PROTOTYPES = {
     "infmoe_serialization_size": (_i32, [_vp, C.POINTER(_sz)]),
     "infmoe_serialize": (_i32, [_vp, _vp, _sz]),
     "infmoe_deserialize": (_i32, [C.c_char_p, _vp, _sz, C.POINTER(_vp)]),
+    "infmoe_npz_read_f32": (_i32, [C.c_char_p, C.c_char_p, _vp, _sz, _sz]),
     "infmoe_last_error": (C.c_char_p, []),
     "infmoe_plugin_name": (C.c_char_p, []),
     "infmoe_plugin_version": (C.c_char_p, []),

@@ -6,6 +6,7 @@
 #include "../../include/infmoe.h"
 #include "kernels/kernels.h"
 #include "moe_layer.h"
+#include "npz_reader.h"
 #include "sublayers/t5ff_layer.h"
 
 using namespace infmoe;
@@ -233,6 +234,15 @@ int32_t infmoe_deserialize(const char* layer_name, const void* data, size_t byte
         INFMOE_TRY(MoELayer::deserialize(layer_name, data, bytes, &layer));
         *out = new infmoe_plugin{std::move(layer)};
         return INFMOE_OK;
+    });
+}
+
+int32_t infmoe_npz_read_f32(const char* path, const char* name, float* dst_host, size_t rows, size_t cols) {
+    return guarded([&]() -> int32_t {
+        if (path == nullptr || name == nullptr || dst_host == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "null argument");
+        NpzReader npz;
+        INFMOE_TRY(npz.open(path));
+        return npz.read_f32(name, dst_host, rows, cols);
     });
 }
 

@@ -180,6 +180,18 @@ Status MoELayer::workspaceSize(const int32_t* dims, int32_t nbDims, size_t* byte
 
 Status MoELayer::initialize() {
     if (mInitialized) return INFMOE_OK;
+    // all or nothing: a failure half way (a weight array that is missing, an allocation that does not
+    // fit) releases what the earlier steps created, so that a retry starts from a clean layer
+    const Status s = initializeSteps();
+    if (s != INFMOE_OK) {
+        const std::string why = last_error_slot();
+        (void)terminate();
+        last_error_slot() = why;
+    }
+    return s;
+}
+
+Status MoELayer::initializeSteps() {
     const int E = mParams.expertCount, d = mParams.embeddingSize;
     INFMOE_TRY(mSublayer->initialize());
     // plugin/MoELayerPlugin.cc:14-26 (done on the first enqueue there)
@@ -337,8 +349,19 @@ Status MoELayer::setTiming(int depth) {
     if (depth < 0 || depth > 4096) return fail(INFMOE_ERR_INVALID_ARGUMENT, "timing depth must be 0..4096");
     if (depth != mTimingDepth) {
         for (auto e : mMarks) (void)hipEventDestroy(e);
-        mMarks.assign((size_t)depth * (INFMOE_N_PHASES + 1), nullptr);
-        for (auto& e : mMarks) INFMOE_HIP(hipEventCreate(&e));
+        mMarks.clear();
+        mTimingDepth = 0;
+        mTiming = false;
+        std::vector<hipEvent_t> marks((size_t)depth * (INFMOE_N_PHASES + 1), nullptr);
+        for (auto& e : marks) {
+            const hipError_t err = hipEventCreate(&e);
+            if (err != hipSuccess) {  // leave timing off rather than half built
+                for (auto m : marks)
+                    if (m) (void)hipEventDestroy(m);
+                return hip_fail(err, "hipEventCreate");
+            }
+        }
+        mMarks.swap(marks);
         mTimingDepth = depth;
     }
     mTiming = depth > 0;
@@ -401,27 +424,40 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     for (int e = 0; e < E; ++e)
         if (count[e] > 0) order.push_back(e);
     std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return count[a] > count[b]; });
-    int k = 0;
-    for (const int e : order) {
-        const int slot = k % mc;
-        char* slotPtr = c.slots + c.slotStride * (size_t)slot;
-        if (k >= mc) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[k - mc], 0));
-        INFMOE_TRY(mSublayer->copyWeights(slotPtr, e, mCopyStream));
-        INFMOE_HIP(hipEventRecord(mCopyDone[k], mCopyStream));
-        hipStream_t cs = mComputeStreams[k % mComputeStreams.size()];
-        INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
-        // rows of different experts are disjoint, so each expert gets its own stretch of the
-        // shared scratch (row stride applied: the public reference omits it at :373,391-392)
-        INFMOE_TRY(mSublayer->run(count[e], slotPtr, c.routed + (size_t)offset[e] * d, c.post + (size_t)offset[e] * d,
-                                  c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
-        INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
-        ++k;
+    // Whatever happens in the loop, the compute streams forked above are joined back into the caller's
+    // stream before returning: an error half way must not leave work that nothing waits for.
+    auto queueExperts = [&]() -> Status {
+        int k = 0;
+        for (const int e : order) {
+            const int slot = k % mc;
+            char* slotPtr = c.slots + c.slotStride * (size_t)slot;
+            if (k >= mc) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[k - mc], 0));
+            INFMOE_TRY(mSublayer->copyWeights(slotPtr, e, mCopyStream));
+            INFMOE_HIP(hipEventRecord(mCopyDone[k], mCopyStream));
+            hipStream_t cs = mComputeStreams[k % mComputeStreams.size()];
+            INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
+            // rows of different experts are disjoint, so each expert gets its own stretch of the
+            // shared scratch (row stride applied: the public reference omits it at :373,391-392)
+            INFMOE_TRY(mSublayer->run(count[e], slotPtr, c.routed + (size_t)offset[e] * d, c.post + (size_t)offset[e] * d,
+                                      c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
+            INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
+            ++k;
+        }
+        return INFMOE_OK;
+    };
+    const Status queued = queueExperts();
+    const std::string why = queued != INFMOE_OK ? last_error_slot() : std::string();
+    // the copy stream's last work is waited for by a compute stream unless the loop broke off in between
+    if (queued != INFMOE_OK) {
+        INFMOE_HIP(hipEventRecord(mFork, mCopyStream));
+        INFMOE_HIP(hipStreamWaitEvent(stream, mFork, 0));
     }
     for (size_t i = 0; i < mComputeStreams.size(); ++i) {
         INFMOE_HIP(hipEventRecord(mJoin[i], mComputeStreams[i]));
         INFMOE_HIP(hipStreamWaitEvent(stream, mJoin[i], 0));
     }
-    return INFMOE_OK;
+    if (queued != INFMOE_OK) last_error_slot() = why;
+    return queued;
 }
 
 Status MoELayer::lastRouting(int32_t* countHost, int32_t* statsHost) {
@@ -501,7 +537,16 @@ Status MoELayer::deserialize(const char* layerName, const void* data, size_t byt
     memcpy(p.centroids.data(), f, 4 * nc);
     p.layernormWeight.resize(nl);
     memcpy(p.layernormWeight.data(), f + 4 * nc, 4 * nl);
-    return create(std::move(p), out);
+    const uint32_t storedFlags = head[8];
+    INFMOE_TRY(create(std::move(p), out));
+    // the flags are a function of the variant string (plugin/MoELayerPlugin.cc:44-58); a blob whose flag
+    // word says otherwise was not written by serialize()
+    const MoEFlags& fl = (*out)->mParams.flags;
+    if (storedFlags != ((fl.layernormOnInputBeforeScore ? 1u : 0u) | (fl.baseLayerOutputMix ? 2u : 0u))) {
+        out->reset();
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "serialized layer: flag word %u does not belong to its moe_variant", storedFlags);
+    }
+    return INFMOE_OK;
 }
 
 }  // namespace infmoe

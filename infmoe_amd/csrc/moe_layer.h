@@ -62,6 +62,7 @@ class MoELayer {
     bool resident() const;
     Status checkDims(const int32_t* dims, int32_t nbDims, int* tokens) const;
     Status runStreamed(int T, const Carve& c, hipStream_t stream);
+    Status initializeSteps();
 
     MoEParams mParams;
     std::shared_ptr<MoESubLayer> mSublayer;

@@ -37,20 +37,28 @@ Status parse_npy_header(const uint8_t* buf, size_t n, NpyHeader* h) {
     if (hoff + hlen > n) return fail(INFMOE_ERR_IO, "npy header longer than expected");
     const std::string dict(reinterpret_cast<const char*>(buf + hoff), hlen);
     h->data_offset = hoff + hlen;
-    size_t p = dict.find("'descr'");
-    if (p == std::string::npos) return fail(INFMOE_ERR_IO, "npy header without descr");
-    p = dict.find('\'', dict.find(':', p));
+    // value of `key`: position of the first character after "'key' :" and blanks, or npos
+    auto value_of = [&](const char* key) -> size_t {
+        size_t p = dict.find(key);
+        if (p == std::string::npos) return p;
+        p = dict.find(':', p);
+        if (p == std::string::npos) return p;
+        return dict.find_first_not_of(" ", p + 1);
+    };
+    size_t p = value_of("'descr'");
+    if (p == std::string::npos || dict[p] != '\'') return fail(INFMOE_ERR_IO, "npy header without a descr string");
     const size_t q = dict.find('\'', p + 1);
-    if (p == std::string::npos || q == std::string::npos) return fail(INFMOE_ERR_IO, "bad npy descr");
+    if (q == std::string::npos) return fail(INFMOE_ERR_IO, "bad npy descr");
     h->descr = dict.substr(p + 1, q - p - 1);
-    p = dict.find("'fortran_order'");
+    p = value_of("'fortran_order'");
     if (p == std::string::npos) return fail(INFMOE_ERR_IO, "npy header without fortran_order");
-    h->fortran = dict.compare(dict.find_first_not_of(" ", dict.find(':', p) + 1), 4, "True") == 0;
-    p = dict.find("'shape'");
-    if (p == std::string::npos) return fail(INFMOE_ERR_IO, "npy header without shape");
-    p = dict.find('(', p);
+    if (dict.compare(p, 4, "True") == 0) h->fortran = true;
+    else if (dict.compare(p, 5, "False") == 0) h->fortran = false;
+    else return fail(INFMOE_ERR_IO, "bad npy fortran_order");
+    p = value_of("'shape'");
+    if (p == std::string::npos || dict[p] != '(') return fail(INFMOE_ERR_IO, "npy header without a shape tuple");
     const size_t e = dict.find(')', p);
-    if (p == std::string::npos || e == std::string::npos) return fail(INFMOE_ERR_IO, "bad npy shape");
+    if (e == std::string::npos) return fail(INFMOE_ERR_IO, "bad npy shape");
     uint64_t v = 0;
     bool in_num = false;
     for (size_t i = p + 1; i <= e; ++i) {
@@ -106,6 +114,9 @@ Status NpzReader::open(const char* path) {
         if (rd32(r) != kSigEocd64) return fail(INFMOE_ERR_IO, "%s: bad zip64 end record", mPath.c_str());
         n_entries = rd64(r + 32), cd_size = rd64(r + 40), cd_off = rd64(r + 48);
     }
+    if (cd_off > fsize || cd_size > fsize - cd_off)
+        return fail(INFMOE_ERR_IO, "%s: central directory lies outside the file", mPath.c_str());
+    mFileSize = fsize;
     std::vector<uint8_t> cd((size_t)cd_size);
     INFMOE_TRY(read_at(cd_off, cd.data(), cd.size()));
     size_t p = 0;
@@ -147,7 +158,8 @@ std::vector<std::string> NpzReader::names() const {
     return v;
 }
 
-Status NpzReader::read_f32(const char* name_in, float* dst, size_t count) {
+Status NpzReader::read_f32(const char* name_in, float* dst, size_t rows, size_t cols) {
+    const size_t count = rows * (cols ? cols : 1);
     std::string name(name_in);
     if (name.size() > 4 && name.compare(name.size() - 4, 4, ".npy") == 0) name.resize(name.size() - 4);
     auto it = mEntries.find(name);
@@ -157,6 +169,9 @@ Status NpzReader::read_f32(const char* name_in, float* dst, size_t count) {
     INFMOE_TRY(read_at(en.local_offset, lh, sizeof(lh)));
     if (rd32(lh) != kSigLocal) return fail(INFMOE_ERR_IO, "%s: bad local header for %s", mPath.c_str(), name.c_str());
     const uint64_t data_off = en.local_offset + 30 + rd16(lh + 26) + rd16(lh + 28);
+    if (data_off > mFileSize || en.comp_size > mFileSize - data_off)
+        return fail(INFMOE_ERR_IO, "%s: member %s lies outside the file", mPath.c_str(), name.c_str());
+    if (en.uncomp_size > ((uint64_t)1 << 40)) return fail(INFMOE_ERR_IO, "%s: member %s is implausibly large", mPath.c_str(), name.c_str());
 
     std::vector<uint8_t> raw;  // the uncompressed member (header + data) when deflated
     NpyHeader h;
@@ -198,11 +213,23 @@ Status NpzReader::read_f32(const char* name_in, float* dst, size_t count) {
     if (h.descr != "<f4" && h.descr != "=f4" && h.descr != "|f4" && h.descr != "f4")
         return fail(INFMOE_ERR_IO, "%s: %s has dtype %s, expected little-endian float32", mPath.c_str(), name.c_str(), h.descr.c_str());
     uint64_t elems = 1;
-    for (uint64_t s : h.shape) elems *= s;
-    // the reference asserts on the byte count (plugin/sublayers/T5FFLayer.cc:62,69,76,83)
-    if (elems != count || h.data_offset + elems * 4 > en.uncomp_size)
-        return fail(INFMOE_ERR_INVALID_ARGUMENT, "%s: %s holds %llu floats, expected %zu", mPath.c_str(), name.c_str(),
-                    (unsigned long long)elems, count);
+    std::string shape_text = "(";
+    for (uint64_t s : h.shape) {
+        if (s != 0 && elems > UINT64_MAX / s) return fail(INFMOE_ERR_IO, "%s: %s has an overflowing shape", mPath.c_str(), name.c_str());
+        elems *= s;
+        shape_text += std::to_string(s) + ",";
+    }
+    shape_text += ")";
+    // The reference asserts on the byte count only (plugin/sublayers/T5FFLayer.cc:62,69,76,83), so a
+    // matrix saved transposed ([d][h] where [h][d] is meant: same count) passes there; here the shape
+    // has to be the expected one.
+    const bool shape_ok = cols == 0 ? (h.shape.size() == 1 && h.shape[0] == rows)
+                                    : (h.shape.size() == 2 && h.shape[0] == rows && h.shape[1] == cols);
+    if (!shape_ok || elems != count)
+        return fail(INFMOE_ERR_INVALID_ARGUMENT, "%s: %s has shape %s, expected (%zu,%s)", mPath.c_str(), name.c_str(),
+                    shape_text.c_str(), rows, cols ? std::to_string(cols).c_str() : "");
+    if (h.data_offset > en.uncomp_size || elems * 4 > en.uncomp_size - h.data_offset)
+        return fail(INFMOE_ERR_IO, "%s: %s is shorter than its header says", mPath.c_str(), name.c_str());
 
     const bool transpose = h.fortran && h.shape.size() == 2 && h.shape[0] > 1 && h.shape[1] > 1;
     if (h.fortran && h.shape.size() > 2) return fail(INFMOE_ERR_UNSUPPORTED, "%s: Fortran-ordered arrays above 2-D are not supported", name.c_str());

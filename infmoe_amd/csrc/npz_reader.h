@@ -21,9 +21,9 @@ class NpzReader {
     ~NpzReader();
     Status open(const char* path);
     bool has(const char* name) const;
-    // Reads member `name` (with or without the ".npy" suffix) into dst as C-ordered float32;
-    // fails unless it is '<f4' with exactly `count` elements.
-    Status read_f32(const char* name, float* dst, size_t count);
+    // Reads member `name` (with or without the ".npy" suffix) into dst as C-ordered float32; fails
+    // unless it is '<f4' of shape (rows, cols), or (rows,) when cols == 0.
+    Status read_f32(const char* name, float* dst, size_t rows, size_t cols);
     std::vector<std::string> names() const;
 
    private:
@@ -33,6 +33,7 @@ class NpzReader {
     };
     FILE* mFile = nullptr;
     std::string mPath;
+    uint64_t mFileSize = 0;
     std::map<std::string, Entry> mEntries;
     Status read_at(uint64_t off, void* dst, size_t n);
 };

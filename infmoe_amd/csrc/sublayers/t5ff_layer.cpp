@@ -85,25 +85,48 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     return INFMOE_OK;
 }
 
+Status T5FFLayer::loadFromFile() {
+    NpzReader npz;
+    INFMOE_TRY(npz.open(mWeightFile.c_str()));
+    INFMOE_TRY(ensureHostStore());
+    static const char* kGated[] = {"layer_norm_weight", "wi_0_weight", "wi_1_weight", "wo_weight"};
+    static const char* kRelu[] = {"layer_norm_weight", "wi_weight", "wo_weight"};
+    const char* const* keys = mFfnKind == FFN_GATED_GELU ? kGated : kRelu;
+    const size_t d = mEmbeddingSize, h = mHiddenSize;
+    for (int e = 0; e < mExpertCount; ++e) {
+        float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)e);
+        for (int j = 0; j <= nMatrices(); ++j) {
+            size_t off = 0, cnt = 0;
+            keyIndex(keys[j], &off, &cnt);
+            const std::string name = std::to_string(e) + "/" + keys[j];  // README.md:121
+            if (!npz.has(name.c_str())) {
+                // name the likely cause when the file holds the other FFN kind's arrays
+                const std::string other = std::to_string(e) + (mFfnKind == FFN_GATED_GELU ? "/wi_weight" : "/wi_0_weight");
+                if (npz.has(other.c_str()))
+                    return fail(INFMOE_ERR_MISSING_FIELD,
+                                "%s: no array named %s but %s exists: the file holds %s experts; set ffn_kind accordingly",
+                                mWeightFile.c_str(), name.c_str(), other.c_str(),
+                                mFfnKind == FFN_GATED_GELU ? "relu (wi, wo)" : "gated_gelu (wi_0, wi_1, wo)");
+            }
+            // shapes as python/infmoe/config.py:46-52 saves them: gamma (d,), input-side matrices (h, d), wo (d, h)
+            const bool isWo = j == nMatrices();
+            INFMOE_TRY(npz.read_f32(name.c_str(), slot + off, j == 0 ? d : (isWo ? d : h), j == 0 ? 0 : (isWo ? h : d)));
+            mHave[(size_t)e * (nMatrices() + 1) + j] = 1;
+        }
+    }
+    return INFMOE_OK;
+}
+
 Status T5FFLayer::initialize() {
     // plugin/sublayers/T5FFLayer.cc:143-147
     if (mHostWeights == nullptr) {
         if (mWeightFile.empty()) return fail(INFMOE_ERR_STATE, "T5_FF: no expert_weight_file and no weights given by pointer");
-        NpzReader npz;
-        INFMOE_TRY(npz.open(mWeightFile.c_str()));
-        INFMOE_TRY(ensureHostStore());
-        static const char* kGated[] = {"layer_norm_weight", "wi_0_weight", "wi_1_weight", "wo_weight"};
-        static const char* kRelu[] = {"layer_norm_weight", "wi_weight", "wo_weight"};
-        const char* const* keys = mFfnKind == FFN_GATED_GELU ? kGated : kRelu;
-        for (int e = 0; e < mExpertCount; ++e) {
-            float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)e);
-            for (int j = 0; j <= nMatrices(); ++j) {
-                size_t off = 0, cnt = 0;
-                keyIndex(keys[j], &off, &cnt);
-                const std::string name = std::to_string(e) + "/" + keys[j];  // README.md:121
-                INFMOE_TRY(npz.read_f32(name.c_str(), slot + off, cnt));
-                mHave[(size_t)e * (nMatrices() + 1) + j] = 1;
-            }
+        const Status loaded = loadFromFile();
+        if (loaded != INFMOE_OK) {  // leave no half-filled store behind: a retry reads the file again
+            const std::string why = last_error_slot();
+            terminate();
+            last_error_slot() = why;
+            return loaded;
         }
     }
     for (size_t i = 0; i < mHave.size(); ++i)

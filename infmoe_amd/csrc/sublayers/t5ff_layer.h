@@ -55,6 +55,7 @@ class T5FFLayer : public MoESubLayer {
     size_t slotStride() const { return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind)); }
     int keyIndex(const char* key, size_t* offsetFloats, size_t* countFloats) const;
     Status ensureHostStore();
+    Status loadFromFile();
 
     float* mHostWeights = nullptr;   // page-locked, E slots of slotStride() bytes
     std::vector<uint8_t> mHave;      // [E][nMatrices+1] which arrays have been provided
