@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c5|c4|c3|c1] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c5|c4|c3|c1] [--no-cpu] [--no-secondary]
 
 A step is one infmoe_enqueue over one batch of synthetic input that is already resident in
 HBM.  The default workload is the configuration the headline metric is quoted on: cpm_2,
@@ -25,10 +25,14 @@ sys.path.insert(0, ROOT)
 
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+PCIE_PEAK_GBS = 64.0           # host link, PCIe Gen5 x16, one direction
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # benchmark scaled by what the same counters read for the row-copy kernels of known size
 # (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt).  Counters cannot be read from inside a run.
-MEASURED_TRAFFIC_BYTES = {"c2": 5.74e9, "c5": 4.04e9}
+# Kept as the ratio counter bytes / algorithmic bytes of the profiled launch (c2: 5.74 GB against 5.52 GB of
+# weights and activations; c5: 4.04 GB against 4.03 GB of weights of 24 active experts) and applied to the
+# algorithmic bytes of the run at hand, whose number of active experts may differ.
+MEASURED_TRAFFIC_RATIO = {"c2": 5.74 / 5.52, "c5": 4.04 / 4.03}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
@@ -128,6 +132,102 @@ def cpu_baseline(cfg, x, cent, gamma, slots, bias, sample_tokens):
                       f"oracle/moe_cpu.c (FP32, OpenMP, AVX2), {dt:.2f} s"}
 
 
+def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False):
+    """W untimed steps, then K timed ones between two events on the layer's stream, with the library's phase
+    marks (HIP events on the same stream) kept for exactly those K steps."""
+    n_mat = 3 if gated else 2  # weight matrices of an expert
+    E, d, h = cfg["E"], cfg["d"], cfg["h"]
+    B, S = x.shape[0], x.shape[1]
+    T = B * S
+    dims = [B, S, d]
+    ws = torch.empty(plugin.workspace_size(dims), dtype=torch.uint8, device="cuda")
+    y = torch.empty_like(x)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
+
+    plugin.set_timing(steps)  # HIP events at the phase boundaries, kept for every step of the timed region
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t_wall) * 1e3 / steps
+    ms_per_step = start.elapsed_time(end) / steps
+    # per-phase averages over exactly the steps of the timed region (events recorded on the layer's stream)
+    phase_runs = plugin.timing_history(steps)
+    assert len(phase_runs) == steps
+    last = phase_runs[-1]
+    phases = {k: float(np.mean([p[k] for p in phase_runs])) for k in phase_runs[0]}
+    count, stats = plugin.last_routing()
+    active = int((count > 0).sum())
+
+    resident = cfg["mc"] >= E
+    few_rows = T <= 16 * E  # same rule the sub-layer uses to pick the few-row kernels
+    # average launch of the two expert kernels; the gated form's first launch takes two matrices, so its
+    # figures are per matrix: (time of both launches) / 3
+    gemm_ms = (phases["expert_gemm1"] + phases["expert_gemm2"]) / n_mat
+    launches = ("two launches per step: wi_0 and wi_1 with gelu*mul, wo with residual; figures per weight matrix"
+                if gated else "two launches per step: wi with ReLU, wo with residual")
+    if not resident:
+        # streamed experts: the host link bounds the call, not HBM and not the matrix core
+        bytes_per_call = active * 4.0 * (d + n_mat * d * h)
+        roofline = {"bound": "pcie", "achieved": round(bytes_per_call / (phases["expert_gemm1"] * 1e-3) / 1e9, 2),
+                    "peak": PCIE_PEAK_GBS, "unit": "GB/s", "traffic": None,
+                    "kernel": "host-to-device expert copies overlapped with expert kernels",
+                    "note": "bounded by the host link (PCIe Gen5 x16, 64 GB/s per direction): achieved = streamed weight "
+                            "bytes / expert-loop time"}
+    elif few_rows:
+        bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
+        roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "traffic": None if gated or name not in MEASURED_TRAFFIC_RATIO
+                    else round(MEASURED_TRAFFIC_RATIO[name] * bytes_per_launch),
+                    "kernel": f"expert_skinny_kernel ({launches})",
+                    "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
+    else:
+        flops_per_launch = 2.0 * T * d * h
+        roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
+                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "traffic": None if gated or name not in MEASURED_TRAFFIC_RATIO
+                    else round(MEASURED_TRAFFIC_RATIO[name] * 4.0 * (E * d * h + T * d + T * h)),
+                    "kernel": f"expert_gemm_grouped_kernel ({launches})",
+                    "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
+    roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+
+    # the bandwidth-bound phases: algorithmic bytes / phase time (the phase times include the launch
+    # gaps and the event marks, a few microseconds each), against the HBM peak
+    cpm2 = cfg["variant"] == "cpm_2"
+    mix = cfg["variant"] == "base_layer"
+    phase_bytes = {
+        "gating": 4.0 * (T * d + E * d + (d if cpm2 else 0) + 2 * T),
+        "scatter": 4.0 * (2 * T * d + T + (2 * T if mix else 0)),
+        "expert_norm": 4.0 * (2 * T * d + d),
+        "gather": 4.0 * ((3 * T * d + 2 * T) if mix else (2 * T * d + T)),
+    }
+    phase_rates = {k: {"bytes": v, "GB/s": round(v / (phases[k] * 1e-3) / 1e9, 1),
+                       "frac_of_hbm_peak": round(v / (phases[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                   for k, v in phase_bytes.items() if phases.get(k, 0) > 0}
+    return dict(ms_per_step=ms_per_step, wall_ms=wall_ms, phases=phases, last=last, count=count, stats=stats,
+                active=active, resident=resident, roofline=roofline, phase_rates=phase_rates, tokens=T)
+
+
+def secondary_line(m, cfg, name):
+    """What the headline line says of the primary workload, shortened, for a further workload of the same run."""
+    return {"workload": f"{name}: {cfg['variant']} E={cfg['E']} d={cfg['d']} h={cfg['h']} tokens={m['tokens']}",
+            "value": round(m["tokens"] / (m["ms_per_step"] * 1e-3), 1), "unit": "tokens/s",
+            "ms_per_step": round(m["ms_per_step"], 4), "active_experts": m["active"],
+            "tokens_per_expert_min_max": [int(m["count"].min()), int(m["count"].max())],
+            "roofline": m["roofline"], "phases_ms": {k: round(v, 4) for k, v in m["phases"].items()},
+            "phase_rates": m["phase_rates"]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,6 +239,8 @@ def main():
     ap.add_argument("--ffn", default="relu", choices=["relu", "gated_gelu"],
                     help="relu: the two-matrix form the headline metric is quoted on; gated_gelu: the three-matrix "
                          "form (an extra measurement, without the CPU leg)")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="with the default workload: do not also measure the decode shape (c5) and the skewed one (c4)")
     ap.add_argument("--replicate-weights", action="store_true",
                     help="profiling aid: give every expert the values of expert 0 (short set-up, same work)")
     args = ap.parse_args()
@@ -163,78 +265,10 @@ def main():
     torch.cuda.set_device(0)
     plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=not args.no_cpu,
                                                       replicate=args.replicate_weights)
-    dims = [B, S, d]
-    ws = torch.empty(plugin.workspace_size(dims), dtype=torch.uint8, device="cuda")
-    y = torch.empty_like(x)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def step():
-        plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
-
-    plugin.set_timing(args.steps)  # HIP events at the phase boundaries, kept for every step of the timed region
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t_wall = time.perf_counter()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(args.steps):
-        step()
-    end.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t_wall) * 1e3 / args.steps
-    ms_per_step = start.elapsed_time(end) / args.steps
-    # per-phase averages over exactly the steps of the timed region (events recorded on the layer's stream)
-    phase_runs = plugin.timing_history(args.steps)
-    assert len(phase_runs) == args.steps
-    last = phase_runs[-1]
-    phases = {k: float(np.mean([p[k] for p in phase_runs])) for k in phase_runs[0]}
-    count, stats = plugin.last_routing()
-    active = int((count > 0).sum())
-
-    resident = cfg["mc"] >= E
-    few_rows = T <= 16 * E  # same rule the sub-layer uses to pick the few-row kernels
-    # average launch of the two expert kernels; the gated form's first launch takes two matrices, so its
-    # figures are per matrix: (time of both launches) / 3
-    gemm_ms = (phases["expert_gemm1"] + phases["expert_gemm2"]) / n_mat
-    launches = ("two launches per step: wi_0 and wi_1 with gelu*mul, wo with residual; figures per weight matrix"
-                if gated else "two launches per step: wi with ReLU, wo with residual")
-    if not resident:
-        # streamed experts: the host link bounds the call; report the achieved copy rate
-        bytes_per_call = active * 4.0 * (d + n_mat * d * h)
-        roofline = {"bound": "hbm", "achieved": round(bytes_per_call / (phases["expert_gemm1"] * 1e-3) / 1e9, 2),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": None,
-                    "kernel": "host-to-device expert copies overlapped with expert kernels",
-                    "note": "bounded by the host link (PCIe), not by HBM: achieved = streamed weight bytes / expert-loop time"}
-    elif few_rows:
-        bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
-        roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "traffic": None if gated else MEASURED_TRAFFIC_BYTES.get(args.config),
-                    "kernel": f"expert_skinny_kernel ({launches})",
-                    "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
-    else:
-        flops_per_launch = 2.0 * T * d * h
-        roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
-                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "traffic": None if gated else MEASURED_TRAFFIC_BYTES.get(args.config),
-                    "kernel": f"expert_gemm_grouped_kernel ({launches})",
-                    "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
-    roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
-
-    # the bandwidth-bound phases: algorithmic bytes / phase time (the phase times include the launch
-    # gaps and the event marks, a few microseconds each), against the HBM peak
-    cpm2 = cfg["variant"] == "cpm_2"
-    mix = cfg["variant"] == "base_layer"
-    phase_bytes = {
-        "gating": 4.0 * (T * d + E * d + (d if cpm2 else 0) + 2 * T),
-        "scatter": 4.0 * (2 * T * d + T + (2 * T if mix else 0)),
-        "expert_norm": 4.0 * (2 * T * d + d),
-        "gather": 4.0 * ((3 * T * d + 2 * T) if mix else (2 * T * d + T)),
-    }
-    phase_rates = {k: {"bytes": v, "GB/s": round(v / (phases[k] * 1e-3) / 1e9, 1),
-                       "frac_of_hbm_peak": round(v / (phases[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
-                   for k, v in phase_bytes.items() if phases.get(k, 0) > 0}
+    m = measure(torch, plugin, cfg, args.config, x, args.steps, args.warmup, gated)
+    count, stats, active, resident = m["count"], m["stats"], m["active"], m["resident"]
+    ms_per_step, wall_ms, phases, last = m["ms_per_step"], m["wall_ms"], m["phases"], m["last"]
+    roofline, phase_rates = m["roofline"], m["phase_rates"]
 
     out = {
         "metric": f"MoE-layer tokens/s (E={E},d={d},h={h},fp32)",
@@ -262,7 +296,27 @@ def main():
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, x, cent, gamma, slots, bias, min(args.cpu_sample, T))
+    # Further workloads of the same run (the headline `value` above is untouched by them):
+    #   c5, the decode shape: same layer (E, d, h as c2), 64 tokens of the same batch
+    #   c4, the skewed base_layer workload: a layer of its own, built after the first is released
+    secondary = {}
+    if args.config == "c2" and not args.no_secondary and not gated:
+        c5 = dict(CONFIGS["c5"], ffn=args.ffn)
+        x5 = x.reshape(T, d)[:64].reshape(64, 1, d).contiguous()
+        secondary["c5"] = secondary_line(measure(torch, plugin, c5, "c5", x5, max(args.steps, 50), args.warmup), c5, "c5")
     plugin.terminate()
+    plugin.destroy()
+    del slots
+    if args.config == "c2" and not args.no_secondary and not gated:
+        try:
+            c4 = dict(CONFIGS["c4"], ffn=args.ffn)
+            p4, x4, *_ = build_layer(torch, c4, keep_host=False)
+            secondary["c4"] = secondary_line(measure(torch, p4, c4, "c4", x4.contiguous(), args.steps, args.warmup), c4, "c4")
+            p4.terminate()
+        except Exception as exc:  # the headline line must not depend on the extras
+            secondary["c4"] = {"error": repr(exc)}
+    if secondary:
+        out["secondary"] = secondary
     print(json.dumps(out))
 
 
