@@ -39,7 +39,8 @@ typedef enum infmoe_status {
     INFMOE_ERR_IO = 5,               /* weight file missing / malformed: plugin/MoELayerPluginCreator.cc:132-140 */
     INFMOE_ERR_STATE = 6,            /* call order violated (e.g. enqueue before initialize) */
     INFMOE_ERR_HIP = 7,              /* a HIP runtime call failed (plugin/utility.h:13-21 exits instead) */
-    INFMOE_ERR_NAN = 8               /* a token had no orderable score (plugin/cuda/moe.cu:70,184 assert instead) */
+    INFMOE_ERR_NAN = 8               /* a token had no orderable score (plugin/cuda/moe.cu:70,184 assert instead);
+                                        see infmoe_enqueue for when it is reported */
 } infmoe_status;
 
 /* Same numeric values as nvinfer1::PluginFieldType so a caller can pass fields through. */
@@ -116,7 +117,16 @@ int32_t infmoe_initialize(infmoe_plugin* p);
  * Replaces MoELayerPlugin::enqueue (plugin/MoELayerPlugin.cc:279-416).
  * inputs[0]: device float [B,S,d]; outputs[0]: device float [B,S,d]; `workspace`: device,
  * at least infmoe_workspace_size bytes, 256-byte aligned; `hip_stream`: hipStream_t.
- * Allocates nothing.
+ * Allocates no device memory (the streamed schedule builds a short list of experts on the host heap).
+ *
+ * A token whose scores cannot be ordered (a NaN in its row; the reference asserts there,
+ * plugin/cuda/moe.cu:70,184) does not stop the call, whatever the schedule: the call completes, that
+ * token's output row is NaN in full, every other row is computed as usual, and the token is counted
+ * in stats[1] of infmoe_last_routing.  INFMOE_ERR_NAN is returned once per such call, by whichever
+ * of these comes first: the call itself when it waits for the routing anyway (experts streamed,
+ * max_concurrency < expert_count); the first later infmoe_enqueue on the handle that finds the
+ * device's report (that call returns the code and queues nothing); not at all if infmoe_last_routing
+ * has reported the count in between.
  */
 int32_t infmoe_enqueue(infmoe_plugin* p, const int32_t* dims, int32_t nb_dims, const void* const* inputs,
                        void* const* outputs, void* workspace, void* hip_stream);
@@ -185,10 +195,12 @@ enum { INFMOE_FFN_RELU = 0, INFMOE_FFN_GATED_GELU = 1 };
  * x [T][d]; centroids [E][d]; gamma [d] or NULL (norm_kind NONE); score_bias [E] or NULL;
  * sel int32 [T]; coeff float [T] (the winning score); stats int32[3] as infmoe_last_routing
  * (accumulated with atomics: zero it first) or NULL.
- * `scratch`: NULL, or infmoe_gate_top1_scratch_bytes(T,d,E) bytes (may be 0) of device memory (16-byte aligned,
- * any contents): with it a call with few tokens spreads each token group's embedding dimension
- * over several workgroups, which the reference's cuBLAS call does inside the library.  The result
- * does not depend on it beyond FP32 rounding of the scores.
+ * `scratch`: NULL, or infmoe_gate_top1_scratch_bytes(T,d,E) bytes of device memory (16-byte aligned,
+ * any contents): with it the embedding dimension is cut into slices that different workgroups
+ * take (the reference's cuBLAS call does the like inside the library) - for few tokens so that the
+ * whole chip works, for many so that a slice of the centroids stays in on-chip memory - and a second
+ * launch adds the slices' partial scores.  The result does not depend on it beyond FP32 rounding of
+ * the scores.
  */
 size_t infmoe_gate_top1_scratch_bytes(int32_t T, int32_t d, int32_t E);
 int32_t infmoe_gate_top1(int32_t T, int32_t d, int32_t E, const float* x, const float* centroids, const float* gamma,

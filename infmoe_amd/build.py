@@ -27,6 +27,7 @@ SOURCES = [
     "kernels/expert_gemm_one_gated.hip",
     "kernels/expert_gemm.hip",
     "kernels/gating.hip",
+    "kernels/gating_slab.hip",
     "kernels/expert_skinny.hip",
     "sublayers/t5ff_layer.cpp",
     "npz_reader.cpp",

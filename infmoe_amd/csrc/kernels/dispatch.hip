@@ -274,11 +274,17 @@ __global__ __launch_bounds__(kThreads) void scatter_kernel(int T, int d, const f
 
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void gather_kernel(int T, int d, const float* __restrict__ buf,
-                                                          const int* __restrict__ pos, float* __restrict__ out) {
+                                                          const int* __restrict__ pos, float* __restrict__ out,
+                                                          const float* __restrict__ routed_coeff) {
     const int lane = threadIdx.x & 63;
     const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (r >= T) return;
-    copy_row<VEC>(out + (size_t)pos[r] * d, buf + (size_t)r * d, d, lane);
+    float* dst = out + (size_t)pos[r] * d;
+    if (routed_coeff != nullptr && isnan(routed_coeff[r])) {  // a token the gating could not score: NaN out
+        for (int k = lane; k < d; k += 64) dst[k] = __builtin_nanf("");
+        return;
+    }
+    copy_row<VEC>(dst, buf + (size_t)r * d, d, lane);
 }
 
 template <bool VEC>
@@ -416,12 +422,13 @@ hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, cons
     return hipGetLastError();
 }
 
-hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream) {
+hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream,
+                         const float* routed_coeff) {
     if (T <= 0) return hipSuccess;
     if (vec_ok(d, {buf, out}))
-        gather_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out);
+        gather_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out, routed_coeff);
     else
-        gather_kernel<false><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out);
+        gather_kernel<false><<<row_grid(T), kThreads, 0, stream>>>(T, d, buf, pos, out, routed_coeff);
     return hipGetLastError();
 }
 

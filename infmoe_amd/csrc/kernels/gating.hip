@@ -78,6 +78,7 @@ struct GateArgs {
     int mode;       // GateMode
     int slices;     // workgroups per token group
     int steps_per;  // K chunks per slice
+    int* nan_flag;    // null, or an int (host memory the device can write) set to 1 when a token has no orderable score
     float* partials;  // [slices][T][E + 2]: dot products, row sum, row sum of squares
     float* gpart;     // [groups][slices][2E]: sum and sum of squares of the folded centroid slice
 };
@@ -501,8 +502,9 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg)
             const int I = s_besti[tid];
             if (I < 0) {  // no orderable score: the reference asserts (plugin/cuda/moe.cu:70)
                 sel[t] = 0;
-                coeff[t] = B;
+                coeff[t] = __builtin_nanf("");  // marks the row: the combine step writes NaN for it
                 if (stats) atomicAdd(&stats[1], 1);
+                if (arg.nan_flag) *reinterpret_cast<volatile int*>(arg.nan_flag) = 1;
             } else {
                 sel[t] = I;
                 coeff[t] = B;
@@ -725,6 +727,35 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg)
     }
 }
 
+// centroids * gamma and, per expert, the sum and the Euclidean norm of that product: what
+// fold_centroids_host computes, for callers that hand over the plain centroids on every call.
+__global__ __launch_bounds__(kThreads) void fold_centroids_kernel(int d, int E, const float* __restrict__ C,
+                                                                  const float* __restrict__ gamma,
+                                                                  float* __restrict__ folded, float* __restrict__ cstats) {
+    __shared__ double s_red[kWaves][2];
+    const int e = blockIdx.x, tid = threadIdx.x;
+    double sum = 0.0, sq = 0.0;
+    for (int k = tid; k < d; k += kThreads) {
+        const float v = gamma != nullptr ? C[(size_t)e * d + k] * gamma[k] : C[(size_t)e * d + k];
+        folded[(size_t)e * d + k] = v;
+        sum += v;
+        sq += (double)v * v;
+    }
+    sum = wave_sum(sum);
+    sq = wave_sum(sq);
+    if ((tid & 63) == 0) s_red[tid >> 6][0] = sum, s_red[tid >> 6][1] = sq;
+    __syncthreads();
+    if (tid == 0) {
+        double a = 0.0, b = 0.0;
+        for (int w = 0; w < kWaves; ++w) a += s_red[w][0], b += s_red[w][1];
+        cstats[e] = (float)a;
+        cstats[E + e] = (float)sqrt(b);
+    }
+}
+
+// floats at the end of the scratch that hold the folded centroids and their statistics
+size_t gate_fold_floats(int d, int E) { return (((size_t)E * d + 3) & ~(size_t)3) + (((size_t)2 * E + 3) & ~(size_t)3); }
+
 // How a call is split into workgroups.
 struct GatePlan {
     int mb;         // 16-token blocks per workgroup: 1 or 4
@@ -764,8 +795,12 @@ GatePlan gate_plan(int T, int d, int E, bool vec, size_t scratch_floats) {
     return wide;
 }
 
+// Which launches of a sliced call are issued here: the slices' partial scores may already be in a.partials
+// (written by the slab launch), and the combine may be left to the wave-per-four-tokens kernel.
+enum : int { kLaunchSlices = 1, kLaunchCombine = 2 };
 template <int NBLK>
-hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const GatePlan& plan, hipStream_t stream) {
+hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const GatePlan& plan, hipStream_t stream,
+                       int what = kLaunchSlices | kLaunchCombine) {
     a.slices = plan.slices, a.steps_per = plan.steps_per;
     const dim3 block(kThreads);
     hipError_t err = hipSuccess;
@@ -780,9 +815,11 @@ hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const Gat
             gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups), block, lds, stream>>>(a);                     \
         } else {                                                                                                  \
             a.mode = GATE_SLICES;                                                                                 \
-            gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups * plan.slices), block, lds, stream>>>(a);       \
+            if (what & kLaunchSlices)                                                                             \
+                gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups * plan.slices), block, lds, stream>>>(a);   \
             a.mode = GATE_COMBINE; /* does not touch the staging tile */                                          \
-            gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups), block, 0, stream>>>(a);                       \
+            if (what & kLaunchCombine)                                                                            \
+                gate_top1_kernel<NBLK, M, V, G, P><<<dim3(plan.groups), block, 0, stream>>>(a);                   \
         }                                                                                                         \
     } while (0)
 #define INFMOE_GATE_M(V, G, P)                     \
@@ -807,10 +844,11 @@ hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const Gat
 
 }  // namespace
 
-size_t gate_scratch_floats(int T, int d, int E) {
-    // Enough for every call of up to T tokens.  Only 16-token workgroups are sliced, and only while
-    // there are fewer than kTargetGroups token groups: slices * tokens <= (kTargetGroups / groups + 1)
-    // * groups * 16 <= 16 * kTargetGroups + tokens + 16, and groups * slices <= 2 * kTargetGroups.
+// Scratch of the sliced one-kernel path: enough for every call of up to T tokens.  Only 16-token workgroups
+// are sliced, and only while there are fewer than kTargetGroups token groups: slices * tokens <=
+// (kTargetGroups / groups + 1) * groups * 16 <= 16 * kTargetGroups + tokens + 16, and groups * slices <=
+// 2 * kTargetGroups.
+static size_t sliced_scratch_floats(int T, int d, int E) {
     const int kc = gate_kc(nblk_for(E), 1);
     const size_t W = (size_t)E + 2;
     const size_t max_slices = std::min<size_t>(std::min(kMaxSlices, (d + kc - 1) / kc), std::max<size_t>(1, (size_t)d / (2 * W)));
@@ -820,29 +858,77 @@ size_t gate_scratch_floats(int T, int d, int E) {
     return rows * W + (size_t)2 * kTargetGroups * 2 * (size_t)E;
 }
 
+// [partial scores of either path | folded centroids and their statistics (used when the caller did not fold)]
+size_t gate_scratch_floats(int T, int d, int E) {
+    if (T <= 0) return 0;
+    const size_t partial = std::max(sliced_scratch_floats(T, d, E), gate_slab_scratch_floats(T, d, E));
+    return ((partial + 3) & ~(size_t)3) + gate_fold_floats(d, E);
+}
+
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids, const float* centroid_stats,
-                            float* scratch, size_t scratch_floats) {
-    if (T <= 0) return hipSuccess;
+                            float* scratch, size_t scratch_floats, bool zero_stats, int* nan_flag) {
+    if (T <= 0) return zero_stats && stats ? launch_fill_i32(stats, 4, 0, stream) : hipSuccess;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(centroids) |
                            reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(folded_centroids)) & 15) == 0;
-    const bool pre = folded_centroids != nullptr && centroid_stats != nullptr;
+    bool pre = folded_centroids != nullptr && centroid_stats != nullptr;
     const bool vec = d % 4 == 0 && aligned;
     const bool use_gamma = norm_kind != NORM_NONE && gamma != nullptr;
-    const GatePlan plan = gate_plan(T, d, E, vec, scratch != nullptr ? scratch_floats : 0);
+    // the end of the scratch is set aside for the folded centroids; the partial scores get the rest
+    const size_t fold_floats = gate_fold_floats(d, E);
+    size_t partial_floats = 0;
+    if (scratch != nullptr && scratch_floats >= fold_floats) {
+        partial_floats = scratch_floats - fold_floats;
+        if (!pre && vec) {  // the caller holds plain centroids: fold them here, once per call
+            float* folded = scratch + partial_floats;
+            float* cstats = folded + (((size_t)E * d + 3) & ~(size_t)3);
+            fold_centroids_kernel<<<E, kThreads, 0, stream>>>(d, E, centroids, use_gamma ? gamma : nullptr, folded, cstats);
+            folded_centroids = folded, centroid_stats = cstats;
+            pre = true;
+        }
+    }
     GateArgs a{};
     a.T = T, a.d = d, a.E = E;
     a.X = x, a.C = centroids, a.gamma = gamma, a.Cf = folded_centroids, a.cstats = centroid_stats;
     a.norm_kind = norm_kind, a.bias = score_bias, a.sel = sel, a.coeff = coeff, a.stats = stats;
+    a.nan_flag = nan_flag;
     a.partials = scratch;
-    a.gpart = scratch ? scratch + (size_t)plan.slices * T * (E + 2) : nullptr;
-    switch (nblk_for(E)) {
-        case 1: return launch_nblk<1>(a, vec, pre, use_gamma, plan, stream);
-        case 2: return launch_nblk<2>(a, vec, pre, use_gamma, plan, stream);
-        case 4: return launch_nblk<4>(a, vec, pre, use_gamma, plan, stream);
-        default: return launch_nblk<8>(a, vec, pre, use_gamma, plan, stream);
+    GatePlan plan{};
+    GateSlabPlan slab{};
+    const bool use_slab = pre && vec && gate_slab_plan(T, d, E, partial_floats, &slab);
+    if (use_slab) {
+        // many tokens: partial scores per slice with the centroid slice resident in LDS, then the combine
+        const hipError_t err = launch_gate_slab(slab, T, d, E, x, folded_centroids, scratch, stream,
+                                                zero_stats ? stats : nullptr);
+        if (err != hipSuccess) return err;
+        plan.mb = T < 64 * kTargetGroups ? 1 : 4;
+        plan.groups = (T + 16 * plan.mb - 1) / (16 * plan.mb);
+        plan.slices = slab.slices;
+        plan.steps_per = 0;  // the combine does not walk the embedding dimension
+    } else {
+        plan = gate_plan(T, d, E, vec, partial_floats);
+        if (zero_stats && stats != nullptr) {
+            const hipError_t err = launch_fill_i32(stats, 4, 0, stream);
+            if (err != hipSuccess) return err;
+        }
     }
+    a.gpart = scratch ? scratch + (size_t)plan.slices * T * (E + 2) : nullptr;
+    // a sliced call whose centroids are folded leaves the second launch to the lean combine kernel
+    const bool lean = plan.slices > 1 && pre && vec && gate_combine_ok(d, E);
+    const int what = (use_slab ? 0 : kLaunchSlices) | (lean ? 0 : kLaunchCombine);
+    hipError_t err = hipSuccess;
+    if (what != 0) {
+        switch (nblk_for(E)) {
+            case 1: err = launch_nblk<1>(a, vec, pre, use_gamma, plan, stream, what); break;
+            case 2: err = launch_nblk<2>(a, vec, pre, use_gamma, plan, stream, what); break;
+            case 4: err = launch_nblk<4>(a, vec, pre, use_gamma, plan, stream, what); break;
+            default: err = launch_nblk<8>(a, vec, pre, use_gamma, plan, stream, what); break;
+        }
+    }
+    if (err != hipSuccess || !lean) return err;
+    return launch_gate_combine(T, d, E, plan.slices, scratch, centroid_stats, x, centroids, use_gamma ? gamma : nullptr,
+                               norm_kind, score_bias, sel, coeff, stats, nan_flag, stream);
 }
 
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats) {

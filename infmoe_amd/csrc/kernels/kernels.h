@@ -24,12 +24,46 @@ constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/subla
 // Optional: scratch (gate_scratch_floats(T, d, E) floats, any contents): with it the embedding dimension
 // of a call with few tokens is split over several workgroups per token group, and a second launch adds
 // their partial scores and selects.
+// zero_stats: `stats` (4 ints) is set to zero before anything is counted into it, by the first of two
+// launches where there are two, else by a small fill launch; without it the caller has cleared them.
+// A token without an orderable score (a NaN in its row; the reference asserts, plugin/cuda/moe.cu:70) gets
+// expert 0 and the coefficient NaN, is counted in stats[1], and sets *nan_flag (an int the device can
+// write, e.g. page-locked host memory) to 1 when that pointer is given.
 size_t gate_scratch_floats(int T, int d, int E);
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids = nullptr,
                             const float* centroid_stats = nullptr, float* scratch = nullptr,
-                            size_t scratch_floats = 0);
+                            size_t scratch_floats = 0, bool zero_stats = false, int* nan_flag = nullptr);
+// Calls with many tokens: the first of two launches writes partial scores per slice of the embedding
+// dimension with that slice of the folded centroids resident in LDS (gating_slab.hip); the combine launch
+// of the gating kernel adds the slices and selects.  The plan says how a call is cut; gate_slab_plan
+// returns false for shapes this path does not take (more than 128 experts, d not a multiple of 128, few tokens,
+// scratch too small).
+struct GateSlabPlan {
+    int ks;              // floats of the embedding dimension per slice (a multiple of 128)
+    int slices;          // d / ks, at most kGateMaxSlices
+    int waves;           // waves per workgroup: 4 or 8, each 16 tokens at a time
+    int tiles_per_wave;  // 16-token tiles a wave takes in turn
+    int groups;          // workgroups per slice
+};
+constexpr int kGateMaxSlices = 16;
+constexpr int kGateSlabMinTokens = 1024;
+bool gate_slab_plan(int T, int d, int E, size_t scratch_floats, GateSlabPlan* plan);
+size_t gate_slab_scratch_floats(int T, int d, int E);
+// partials: [slices][T][E + 2] floats (dot products, row sum, row sum of squares)
+// zero_stats: null, or 4 ints that the launch sets to zero (the combine launch counts into them)
+hipError_t launch_gate_slab(const GateSlabPlan& plan, int T, int d, int E, const float* x,
+                            const float* folded_centroids, float* partials, hipStream_t stream,
+                            int* zero_stats = nullptr);
+// The second launch of a sliced gating call: adds the slices' partial scores ([slices][T][E + 2]), selects,
+// and re-scores near ties in float64 from x, the plain centroids and gamma.  Takes up to 128 experts and
+// rows of 16-byte-aligned float4 (gate_combine_ok); centroid_stats as fold_centroids_host makes them.
+bool gate_combine_ok(int d, int E);
+hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* partials, const float* centroid_stats,
+                               const float* x, const float* centroids, const float* gamma, int norm_kind,
+                               const float* score_bias, int* sel, float* coeff, int* stats, int* nan_flag,
+                               hipStream_t stream);
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)
@@ -84,7 +118,10 @@ hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream);
 // ---- scatter / gather / mix (replaces plugin/cuda/moe.cu:214-258)
 hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, const int* pos, float* routed,
                           float* routed_coeff, hipStream_t stream);
-hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream);
+// routed_coeff: null, or [T]; a routed row whose coefficient is NaN (a token the gating could not score) is
+// written as NaN in full
+hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream,
+                         const float* routed_coeff = nullptr);
 hipError_t launch_mix_gather(int T, int d, const int* pos, const float* routed, const float* post,
                              const float* routed_coeff, float* out, hipStream_t stream);
 

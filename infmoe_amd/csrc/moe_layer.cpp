@@ -212,7 +212,12 @@ Status MoELayer::initializeSteps() {
     const size_t routingInts = (size_t)2 * E + 1 + 4;
     INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mRoutingGpu), sizeof(int32_t) * routingInts));
     INFMOE_HIP(hipMemset(mRoutingGpu, 0, sizeof(int32_t) * routingInts));
-    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mRoutingHost), sizeof(int32_t) * routingInts, hipHostMallocDefault));
+    // page-locked and visible to the device: the last int is the flag the gating sets when it meets a
+    // token without an orderable score (the host reads it without waiting for the device)
+    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mRoutingHost), sizeof(int32_t) * (routingInts + 1), hipHostMallocMapped));
+    mNanFlagHost = mRoutingHost + routingInts;
+    *mNanFlagHost = 0;
+    INFMOE_HIP(hipHostGetDevicePointer(reinterpret_cast<void**>(&mNanFlagDev), mNanFlagHost, 0));
     INFMOE_HIP(hipEventCreateWithFlags(&mRoutingDone, hipEventDisableTiming));
     if (resident()) {
         INFMOE_TRY(mSublayer->makeResident());
@@ -247,6 +252,7 @@ Status MoELayer::terminate() {
     if (mRoutingHost) (void)hipHostFree(mRoutingHost);
     mCentroidsGpu = mLayernormGpu = mScoreBiasGpu = nullptr;
     mRoutingGpu = mRoutingHost = nullptr;
+    mNanFlagHost = mNanFlagDev = nullptr;
     if (mCopyStream) (void)hipStreamDestroy(mCopyStream);
     mCopyStream = nullptr;
     for (auto s : mComputeStreams) (void)hipStreamDestroy(s);
@@ -276,6 +282,13 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     if (inputs == nullptr || outputs == nullptr || inputs[0] == nullptr || outputs[0] == nullptr)
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "null input or output");
     if (T == 0) return INFMOE_OK;
+    // An earlier call met a token without an orderable score (a NaN in its row) and the device has said so
+    // since: reported once, by the first call that sees it; this call queues nothing.
+    if (*static_cast<volatile int32_t*>(mNanFlagHost) != 0) {
+        *static_cast<volatile int32_t*>(mNanFlagHost) = 0;
+        return fail(INFMOE_ERR_NAN, "an earlier infmoe_enqueue on this layer met token(s) with no orderable score (NaN input?); "
+                                    "their output rows are NaN");
+    }
     if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255))
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "workspace must be non-null and 256-byte aligned");
     const int E = mParams.expertCount, d = mParams.embeddingSize;
@@ -296,11 +309,11 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     };
     INFMOE_TRY(mark(0));
     // 0-2. norm (cpm_2: for scoring only), scores, top-1          plugin/MoELayerPlugin.cc:312-345
-    INFMOE_HIP(launch_fill_i32(dStats, 4, 0, stream));
     const bool ln = mParams.flags.layernormOnInputBeforeScore;
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
                                 mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream, mFoldedGpu,
-                                mFoldedGpu + (size_t)E * d, c.gateScratch, gate_scratch_floats(T, d, E)));
+                                mFoldedGpu + (size_t)E * d, c.gateScratch, gate_scratch_floats(T, d, E),
+                                /*zero_stats=*/true, mNanFlagDev));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     const bool grouped = resident();
@@ -329,6 +342,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {
         INFMOE_TRY(mark(4));
+        mNanRowsSeen = 0;
         INFMOE_TRY(runStreamed(T, c, stream));
         INFMOE_TRY(mark(5));
     }
@@ -339,9 +353,13 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     if (mParams.flags.baseLayerOutputMix)
         INFMOE_HIP(launch_mix_gather(T, d, c.pos, c.routed, c.post, c.routedCoeff, y, stream));
     else
-        INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream));
+        INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream, c.routedCoeff));
     INFMOE_TRY(mark(7));
     if (timed) ++mTimedCalls;
+    if (!grouped && mNanRowsSeen > 0) {
+        *static_cast<volatile int32_t*>(mNanFlagHost) = 0;  // reported here, not again by the next call
+        return fail(INFMOE_ERR_NAN, "%d token(s) have no orderable score (NaN input?); their output rows are NaN", mNanRowsSeen);
+    }
     return INFMOE_OK;
 }
 
@@ -410,7 +428,9 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     const int32_t* count = mRoutingHost;
     const int32_t* offset = mRoutingHost + E;
     const int32_t* stats = offset + E + 1;
-    if (stats[1] > 0) return fail(INFMOE_ERR_NAN, "%d token(s) have no orderable score (NaN input?)", stats[1]);
+    // tokens without an orderable score do not stop the call: their rows come out as NaN, and enqueue
+    // reports them when everything is queued (this schedule knows of them now; the resident one later)
+    mNanRowsSeen = stats[1];
 
     INFMOE_HIP(hipEventRecord(mFork, stream));
     INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
@@ -468,6 +488,8 @@ Status MoELayer::lastRouting(int32_t* countHost, int32_t* statsHost) {
     INFMOE_HIP(hipMemcpy(tmp.data(), mRoutingGpu, sizeof(int32_t) * tmp.size(), hipMemcpyDeviceToHost));
     if (countHost) memcpy(countHost, tmp.data(), sizeof(int32_t) * E);
     if (statsHost) memcpy(statsHost, tmp.data() + 2 * E + 1, sizeof(int32_t) * 3);
+    // the caller has now been told of that call's NaN rows (stats[1]): the next enqueue does not repeat it
+    if (tmp[2 * E + 1 + 1] > 0) *static_cast<volatile int32_t*>(mNanFlagHost) = 0;
     return INFMOE_OK;
 }
 

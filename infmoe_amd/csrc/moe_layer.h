@@ -77,6 +77,9 @@ class MoELayer {
     float* mFoldedGpu = nullptr;      // centroids * gating gamma [E][d], then [sum E | norm E]
     int32_t* mRoutingGpu = nullptr;   // [count E | offset E+1 | stats 4]
     int32_t* mRoutingHost = nullptr;  // page-locked mirror
+    int32_t* mNanFlagHost = nullptr;  // in the same allocation: set by the gating kernels, read by the host
+    int32_t* mNanFlagDev = nullptr;   // its device address
+    int mNanRowsSeen = 0;             // streamed schedule: NaN rows of the call in progress
     hipStream_t mCopyStream = nullptr;
     std::vector<hipStream_t> mComputeStreams;
     std::vector<hipEvent_t> mCopyDone, mComputeDone, mJoin;

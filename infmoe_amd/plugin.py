@@ -125,8 +125,12 @@ class Plugin:
             pass
 
     # -- torch convenience -----------------------------------------------------------------
-    def forward(self, x):
-        """x: torch float32 ROCm tensor [B, S, d] -> new tensor of the same shape."""
+    def forward(self, x, check_nan: bool = False):
+        """x: torch float32 ROCm tensor [B, S, d] -> new tensor of the same shape.
+
+        check_nan: wait for the call's routing and raise InfMoEError(ERR_NAN) if a token had no orderable
+        score (a NaN in its row), as the reference asserts (plugin/cuda/moe.cu:70); costs a host wait.
+        Without it such a token's output row is NaN and a later call reports the error once."""
         import torch
         assert x.is_cuda and x.dtype == torch.float32 and x.dim() == 3 and x.is_contiguous()
         dims = list(x.shape)
@@ -136,6 +140,10 @@ class Plugin:
         y = torch.empty_like(x)
         stream = torch.cuda.current_stream(x.device).cuda_stream
         self.enqueue(dims, x.data_ptr(), y.data_ptr(), self._workspace.data_ptr(), stream)
+        if check_nan:
+            _, stats = self.last_routing()
+            if stats["nan_rows"] > 0:
+                raise capi.InfMoEError(capi.ERR_NAN, f"{stats['nan_rows']} token(s) have no orderable score (NaN input?)")
         return y
 
 
