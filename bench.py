@@ -239,6 +239,9 @@ def main():
     ap.add_argument("--ffn", default="relu", choices=["relu", "gated_gelu"],
                     help="relu: the two-matrix form the headline metric is quoted on; gated_gelu: the three-matrix "
                          "form (an extra measurement, without the CPU leg)")
+    ap.add_argument("--sweep-tokens", default="",
+                    help="comma-separated token counts: after the workload proper, the same layer is timed on that many "
+                         "tokens of the batch each (e.g. 256,512,1024,2048 with c2: 8 to 64 rows per expert)")
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: do not also measure the decode shape (c5) and the skewed one (c4)")
     ap.add_argument("--replicate-weights", action="store_true",
@@ -304,6 +307,22 @@ def main():
         c5 = dict(CONFIGS["c5"], ffn=args.ffn)
         x5 = x.reshape(T, d)[:64].reshape(64, 1, d).contiguous()
         secondary["c5"] = secondary_line(measure(torch, plugin, c5, "c5", x5, max(args.steps, 50), args.warmup), c5, "c5")
+    # Few to many rows per expert on the same layer: the expert kernels' achieved weight-byte rate (they are
+    # bound by streaming the weights until an expert has some tens of rows) next to their flop rate
+    if args.sweep_tokens:
+        sweep = {}
+        for n in [int(v) for v in args.sweep_tokens.split(",") if v]:
+            xn = x.reshape(T, d)[:n].reshape(n, 1, d).contiguous()
+            mm = measure(torch, plugin, cfg, None, xn, args.steps, args.warmup, gated)
+            g_ms = (mm["phases"]["expert_gemm1"] + mm["phases"]["expert_gemm2"]) / n_mat
+            sweep[str(n)] = {"ms_per_step": round(mm["ms_per_step"], 4), "tokens_per_s": round(n / (mm["ms_per_step"] * 1e-3), 1),
+                             "active_experts": mm["active"], "rows_per_expert_min_max": [int(mm["count"].min()), int(mm["count"].max())],
+                             "expert_launch_ms": round(g_ms, 4),
+                             "weight_GBs": round(mm["active"] * 4.0 * d * h / (g_ms * 1e-3) / 1e9, 1),
+                             "frac_of_hbm_peak": round(mm["active"] * 4.0 * d * h / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                             "TFLOPs": round(2.0 * n * d * h / (g_ms * 1e-3) / 1e12, 2),
+                             "phases_ms": {k: round(v, 4) for k, v in mm["phases"].items()}}
+        out["sweep_tokens"] = sweep
     plugin.terminate()
     plugin.destroy()
     del slots

@@ -30,6 +30,7 @@ SOURCES = [
     "kernels/gating_slab.hip",
     "kernels/expert_skinny.hip",
     "sublayers/t5ff_layer.cpp",
+    "sublayers/sublayer.cpp",
     "npz_reader.cpp",
     "moe_layer.cpp",
     "c_api.cpp",

@@ -9,6 +9,8 @@
 #include <cstddef>
 #include <cstdint>
 
+#include "../../../include/infmoe_sublayer.h"  // RowTile
+
 namespace infmoe {
 
 enum NormKind : int32_t { NORM_NONE = 0, NORM_RMS = 1, NORM_CENTERED = 2 };
@@ -67,13 +69,8 @@ hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* par
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)
-// Row tile of the grouped expert GEMM: `rows` consecutive routed rows of one expert.
-struct RowTile {
-    int32_t expert;
-    int32_t row0;  // first routed row
-    int32_t rows;  // 1..tile height
-    int32_t pad;
-};
+// (RowTile, the unit of work of the grouped expert GEMM - `rows` consecutive routed rows of one expert -
+// is declared in the public plug-in header.)
 constexpr int kCountBlockTokens = 1024;  // tokens ranked by one workgroup
 size_t expert_count_scratch_bytes(int T, int E);
 constexpr int kXcdCount = 8;    // accelerator dies of an MI355X; workgroup ids are dealt to them round-robin

@@ -56,9 +56,11 @@ Status MoELayer::create(MoEParams&& p, std::unique_ptr<MoELayer>* out) {
         if (!S_ISREG(st.st_mode)) return fail(INFMOE_ERR_IO, "weight file must be a regular file: %s", p.weightFile.c_str());
     }
     std::unique_ptr<MoELayer> layer(new MoELayer());
-    INFMOE_TRY(make_sublayer(p.sublayerType.c_str(), p.expertCount, p.embeddingSize, p.hiddenSize,
-                             p.weightFile.empty() ? nullptr : p.weightFile.c_str(), p.maxConcurrency, p.normKind,
-                             p.ffnKind, &layer->mSublayer));
+    SubLayerConfig sc{};
+    sc.expertCount = p.expertCount, sc.embeddingSize = p.embeddingSize, sc.hiddenSize = p.hiddenSize;
+    sc.maxConcurrency = p.maxConcurrency, sc.weightFile = p.weightFile.empty() ? nullptr : p.weightFile.c_str();
+    sc.normKind = p.normKind, sc.ffnKind = p.ffnKind;
+    INFMOE_TRY(make_sublayer(p.sublayerType.c_str(), sc, &layer->mSublayer));
     layer->mParams = std::move(p);
     *out = std::move(layer);
     return INFMOE_OK;
@@ -191,7 +193,27 @@ Status MoELayer::initialize() {
     return s;
 }
 
+// The launch geometry of the kernels is fixed for the part they are written for: workgroup ids are dealt
+// round-robin to 8 accelerator dies (the row-tile schedule of the grouped expert launch and the slice map of
+// the gating count on it) and one workgroup per compute unit means 256 of them.  A device partitioned
+// differently would still compute the same results but balance badly, so it is refused, loudly.
+static Status check_device_geometry() {
+    int dev = 0, cus = 0, xccs = 0;
+    INFMOE_HIP(hipGetDevice(&dev));
+    INFMOE_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (hipDeviceGetAttribute(&xccs, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        xccs = kXcdCount;  // a runtime that cannot tell: the compute-unit count decides
+    }
+    if (cus != 256 || xccs != kXcdCount)
+        return fail(INFMOE_ERR_UNSUPPORTED,
+                    "device %d has %d compute units in %d accelerator dies; this library schedules for 256 in %d (an MI355X in "
+                    "its single-partition mode)", dev, cus, xccs, kXcdCount);
+    return INFMOE_OK;
+}
+
 Status MoELayer::initializeSteps() {
+    INFMOE_TRY(check_device_geometry());
     const int E = mParams.expertCount, d = mParams.embeddingSize;
     INFMOE_TRY(mSublayer->initialize());
     // plugin/MoELayerPlugin.cc:14-26 (done on the first enqueue there)
@@ -299,7 +321,6 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     int32_t* dCount = mRoutingGpu;
     int32_t* dOffset = dCount + E;
     int32_t* dStats = dOffset + E + 1;
-    mSublayer->setLayerTokenCount(T);
 
     const bool timed = mTiming && !mMarks.empty();
     hipEvent_t* marks = timed ? &mMarks[(size_t)(mTimedCalls % mTimingDepth) * (INFMOE_N_PHASES + 1)] : nullptr;
@@ -458,8 +479,9 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
             INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
             // rows of different experts are disjoint, so each expert gets its own stretch of the
             // shared scratch (row stride applied: the public reference omits it at :373,391-392)
-            INFMOE_TRY(mSublayer->run(count[e], slotPtr, c.routed + (size_t)offset[e] * d, c.post + (size_t)offset[e] * d,
-                                      c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
+            INFMOE_TRY(mSublayer->runInLayer(T, count[e], slotPtr, c.routed + (size_t)offset[e] * d,
+                                             c.post + (size_t)offset[e] * d,
+                                             c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
             INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
             ++k;
         }

@@ -1,32 +1,14 @@
 // Error convention of the library: every fallible host function returns a Status (0 = OK) and
 // leaves a message for infmoe_last_error(); nothing aborts or throws across the C ABI.  The
-// reference prints and exits instead (plugin/utility.h:13-21,41-47).
+// reference prints and exits instead (plugin/utility.h:13-21,41-47).  Status, fail() and the message
+// slot are part of the public plug-in header; this one adds what only the library's own sources use.
 #pragma once
 
 #include <hip/hip_runtime_api.h>
 
-#include <cstdarg>
-#include <cstdint>
-#include <cstdio>
-#include <string>
-
-#include "../../include/infmoe.h"
+#include "../../include/infmoe_sublayer.h"
 
 namespace infmoe {
-
-using Status = int32_t;
-
-std::string& last_error_slot();
-
-inline Status fail(Status code, const char* fmt, ...) {
-    char buf[512];
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(buf, sizeof(buf), fmt, ap);
-    va_end(ap);
-    last_error_slot() = buf;
-    return code;
-}
 
 inline Status hip_fail(hipError_t err, const char* what) {
     return fail(INFMOE_ERR_HIP, "%s: %s", what, hipGetErrorString(err));

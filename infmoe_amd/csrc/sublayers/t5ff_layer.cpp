@@ -3,7 +3,6 @@
 #include <cstring>
 
 #include "../npz_reader.h"
-#include "identity_layer.h"
 
 namespace infmoe {
 
@@ -204,12 +203,15 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
 
 Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                       hipStream_t stream) {
-    // outside a layer call (token count of the call unknown) the expert stands alone
-    const int layerTokens = mLayerTokenCount.load(std::memory_order_relaxed);
-    const bool inLayer = layerTokens > 0;
-    return runOne(tokenCount, inLayer ? layerTokens : tokenCount, inLayer ? mExpertCount : 1,
-                  mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights, static_cast<const float*>(input),
-                  static_cast<float*>(output), workspace, stream);
+    // outside a layer call the expert stands alone: a call of tokenCount tokens over one expert
+    return runOne(tokenCount, tokenCount, 1, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream);
+}
+
+Status T5FFLayer::runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input,
+                             void* output, void* workspace, hipStream_t stream) {
+    return runOne(tokenCount, layerTokens, mExpertCount, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream);
 }
 
 Status T5FFLayer::runGrouped(const GroupedRun& g) {
@@ -242,20 +244,6 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     INFMOE_HIP(launch_expert_gemm_grouped(g2, stride, g.tiles, g.sched, g.maxTiles, g.stream));
     if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g2, stride, g.count, g.offset, mExpertCount, g.stream));
     return INFMOE_OK;
-}
-
-Status make_sublayer(const char* type, int expertCount, int embeddingSize, int hiddenSize, const char* weightFile,
-                     int maxConcurrency, int normKind, int ffnKind, std::shared_ptr<MoESubLayer>* out) {
-    // plugin/MoELayerPlugin.cc:28-41, names from plugin/MoELayerPlugin.h:23-26
-    if (type != nullptr && strcmp(type, "T5_FF") == 0) {
-        *out = std::make_shared<T5FFLayer>(expertCount, embeddingSize, hiddenSize, weightFile, maxConcurrency, normKind, ffnKind);
-        return INFMOE_OK;
-    }
-    if (type != nullptr && strcmp(type, "Identity") == 0) {
-        *out = std::make_shared<IdentityLayer>();
-        return INFMOE_OK;
-    }
-    return fail(INFMOE_ERR_UNSUPPORTED, "unsupported sublayer type: %s", type ? type : "(null)");
 }
 
 }  // namespace infmoe

@@ -32,6 +32,8 @@ class T5FFLayer : public MoESubLayer {
     Status copyWeights(void* dst, int expert, hipStream_t stream) override;
     Status run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                hipStream_t stream) override;
+    Status runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input, void* output,
+                      void* workspace, hipStream_t stream) override;
     Status initialize() override;
     void terminate() override;
 

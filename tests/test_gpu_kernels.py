@@ -210,6 +210,18 @@ def test_t5ff_row_counts(lib, torch_cuda, rows, d, h):
     assert_close(got, O.t5ff_run(x, w, "rms", "relu"), what=f"t5ff rows={rows}")
 
 
+# the benchmark's K (4096 into the first product, 10240 into the second) at the row counts of decode batches of
+# a few hundred tokens: few-row kernel (5), one 16-row unit (12), one unit + two 4-row groups... (24 -> 2 units),
+# three units (48), a 32-row block + a 16-row block + a group (52)
+@pytest.mark.parametrize("rows", [5, 12, 24, 48, 52])
+def test_t5ff_row_counts_at_full_width(lib, torch_cuda, rows):
+    d, h = 4096, 10240
+    w = O.draw_expert(26, 0, d, h, "relu")
+    x = O.draw_inputs(rows, rows, d, 2)[0]
+    got = run_t5ff(lib, torch_cuda, x, w, "rms", "relu")
+    assert_close(got, O.t5ff_run(x, w, "rms", "relu"), what=f"t5ff rows={rows} at {d}x{h}")
+
+
 # the two-matrix form keeps two accumulator sets: tiles of up to 192 rows, taller experts in equal tiles
 @pytest.mark.parametrize("rows", [9, 130, 192, 193, 400])
 def test_t5ff_gated_row_counts(lib, torch_cuda, rows):
