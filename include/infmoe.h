@@ -110,7 +110,9 @@ int32_t infmoe_workspace_size(const infmoe_plugin* p, const int32_t* dims, int32
 /* Replaces initialize (plugin/MoELayerPlugin.cc:197-201 -> plugin/sublayers/T5FFLayer.cc:143-147):
  * loads expert weights into page-locked host memory, uploads centroids / gating gamma, creates
  * streams and events, and, when max_concurrency >= expert_count, uploads every expert once into
- * plugin-owned device memory (the reference re-copies on every enqueue, plugin/MoELayerPlugin.cc:365,385-387). */
+ * plugin-owned device memory (the reference re-copies on every enqueue, plugin/MoELayerPlugin.cc:365,385-387);
+ * otherwise it allocates max_concurrency weight slots, which keep experts between calls (an expert
+ * still in a slot is not copied again). */
 int32_t infmoe_initialize(infmoe_plugin* p);
 
 /*
@@ -144,6 +146,15 @@ void infmoe_destroy(infmoe_plugin* p);
  *   [2] tokens whose assignment was re-derived in float64 inside the gating kernel
  */
 int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stats_host);
+
+/*
+ * How the most recent infmoe_enqueue with streamed experts (max_concurrency < expert_count) got its
+ * experts' weights: *copies = experts copied host-to-device in that call, *hits = experts that ran from a
+ * slot still holding them from an earlier call (either may be NULL).  No counterpart in the reference,
+ * which copies every active expert on every call (plugin/MoELayerPlugin.cc:365,385-387).  Both are 0
+ * when the experts are resident.
+ */
+int32_t infmoe_last_streaming(infmoe_plugin* p, int32_t* copies, int32_t* hits);
 
 /*
  * Phase timing (no counterpart in the reference, which only prints wall time from Python,

@@ -125,6 +125,9 @@ class MoESubLayer {
     virtual Status setWeights(int /*expert*/, const char* /*key*/, const float* /*host*/, size_t /*count*/) {
         return fail(INFMOE_ERR_UNSUPPORTED, "this sub-layer takes no weights");
     }
+    /* A number that changes whenever any expert's weights change after initialize(); the layer then drops
+     * the device copies of experts it has kept from earlier calls. */
+    virtual uint64_t weightsVersion() const { return 0; }
     /* Keep every expert in device memory (called once, from infmoe_initialize, when the experts are not
      * streamed).  The default allocates expertCount() slots of weightSize() bytes (rounded up to 256) and
      * fills them with copyWeights. */

@@ -47,6 +47,7 @@ PROTOTYPES = {
     "infmoe_terminate": (_i32, [_vp]),
     "infmoe_destroy": (None, [_vp]),
     "infmoe_last_routing": (_i32, [_vp, _pi32, _pi32]),
+    "infmoe_last_streaming": (_i32, [_vp, _pi32, _pi32]),
     "infmoe_set_timing": (_i32, [_vp, _i32]),
     "infmoe_timing_history": (_i32, [_vp, _pf, _i32, _pi32]),
     "infmoe_last_timing": (_i32, [_vp, C.POINTER(C.c_float)]),

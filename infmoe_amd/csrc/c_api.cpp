@@ -186,6 +186,13 @@ int32_t infmoe_last_routing(infmoe_plugin* p, int32_t* count_host, int32_t* stat
     });
 }
 
+int32_t infmoe_last_streaming(infmoe_plugin* p, int32_t* copies, int32_t* hits) {
+    return guarded([&]() -> int32_t {
+        INFMOE_TRY(check(p));
+        return p->layer->lastStreaming(copies, hits);
+    });
+}
+
 int32_t infmoe_set_timing(infmoe_plugin* p, int32_t enable) {
     return guarded([&]() -> int32_t {
         INFMOE_TRY(check(p));

@@ -122,7 +122,6 @@ bool MoELayer::resident() const {
 }
 
 struct MoELayer::Carve {
-    char* slots = nullptr;
     size_t slotStride = 0;
     char* subWs = nullptr;
     int32_t *sel = nullptr, *pos = nullptr, *rowExpert = nullptr, *sched = nullptr;
@@ -134,8 +133,10 @@ struct MoELayer::Carve {
     size_t total = 0;
 };
 
-// Workspace layout (every block 256-byte aligned):
-//   streamed experts only: max_concurrency weight slots           (plugin/MoELayerPlugin.cc:243-245)
+// Workspace layout (every block 256-byte aligned).  The max_concurrency weight slots of streamed experts,
+// which the reference carves from the workspace (plugin/MoELayerPlugin.cc:243-245), are device memory of
+// the layer here: they keep experts between calls, which memory that the caller may hand to others between
+// calls cannot.
 //   sub-layer scratch for T rows, shared by all experts because their rows are disjoint
 //     (the reference sizes one full-T scratch per slot, :256-263)
 //   sel[T] pos[T] rowExpert[T] | row tiles | scan scratch | coeff[T] routedCoeff[T] | routed[T][d] | post[T][d]
@@ -150,7 +151,6 @@ Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     };
     const int E = mParams.expertCount, d = mParams.embeddingSize;
     c->slotStride = align_up(mSublayer->weightSize());
-    c->slots = resident() ? nullptr : take(c->slotStride * (size_t)mParams.maxConcurrency);
     c->subWs = take(mSublayer->workspaceSize(T));
     c->sel = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
     c->pos = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
@@ -246,6 +246,10 @@ Status MoELayer::initializeSteps() {
     } else {
         // plugin/MoELayerPlugin.cc:182-195 creates max_concurrency streams; here one copy stream
         // feeds the slots and a few compute streams let consecutive experts overlap
+        const size_t stride = align_up(mSublayer->weightSize());
+        INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mSlotPool), stride * (size_t)mParams.maxConcurrency));
+        mSlotExpert.assign(mParams.maxConcurrency, -1);
+        mSlotVersion = mSublayer->weightsVersion();
         INFMOE_HIP(hipStreamCreateWithFlags(&mCopyStream, hipStreamNonBlocking));
         mComputeStreams.resize(std::min(mParams.maxConcurrency, 4));
         for (auto& s : mComputeStreams) INFMOE_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
@@ -277,6 +281,9 @@ Status MoELayer::terminate() {
     mNanFlagHost = mNanFlagDev = nullptr;
     if (mCopyStream) (void)hipStreamDestroy(mCopyStream);
     mCopyStream = nullptr;
+    if (mSlotPool) (void)hipFree(mSlotPool);
+    mSlotPool = nullptr;
+    mSlotExpert.clear();
     for (auto s : mComputeStreams) (void)hipStreamDestroy(s);
     mComputeStreams.clear();
     for (auto* v : {&mCopyDone, &mComputeDone, &mJoin}) {
@@ -436,11 +443,19 @@ Status MoELayer::lastTiming(float* ms) {
 // Experts streamed through max_concurrency device slots (plugin/MoELayerPlugin.cc:360-402).
 // The host learns the token counts once (one blocking copy of E integers), then queues every
 // copy and every expert without blocking again:
-//   copy stream:   [wait: expert k-mc done] copy expert k into slot k % mc, signal copyDone[k]
-//   compute k%n:   [wait: copyDone[k]] run expert k from its slot,          signal computeDone[k]
-// so up to mc-1 experts are prefetched while one computes (the reference prefetches one), and
-// max_concurrency = 1 degenerates to copy, compute, copy, ... with no overlap.  Experts run in
-// descending order of their row counts.
+//   copy stream:   [wait: the slot's previous expert done] copy expert into its slot, signal copyDone[k]
+//   compute k%n:   [wait: copyDone[k]] run expert k from its slot,                     signal computeDone[k]
+// so experts are prefetched while others compute (the reference prefetches one), and
+// max_concurrency = 1 degenerates to copy, compute, copy, ... with no overlap.
+//
+// The slots are the layer's own device memory and keep their contents between calls, each slot
+// remembering which expert it holds (the reference copies every active expert on every call,
+// plugin/MoELayerPlugin.cc:365,385-387).  An expert that is still in a slot from an earlier call runs
+// from there without a copy.  When the experts a call needs do not all fit, the ones already present
+// with the most rows are retained, up to max_concurrency less the two slots the others are streamed
+// through (copy of one under the compute of the other); the rest are copied, most rows first.  A change of
+// any expert's weights (infmoe_set_expert_weights) empties the slots.  Which expert sits where has no
+// influence on the arithmetic: the output is the same bit for bit.
 Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
     const size_t routingInts = (size_t)2 * E + 1 + 4;
@@ -456,33 +471,69 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     INFMOE_HIP(hipEventRecord(mFork, stream));
     INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
     for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
+    if (mSublayer->weightsVersion() != mSlotVersion) {  // some expert's weights changed: nothing cached is valid
+        std::fill(mSlotExpert.begin(), mSlotExpert.end(), -1);
+        mSlotVersion = mSublayer->weightsVersion();
+    }
     // Empty experts are skipped (:361-363,383-384).  The reference takes the others in ascending
     // index; here the ones with most rows go first (stable, so equal counts stay ascending): every
     // expert costs the same copy, and the compute that nothing can hide is the last expert's, so it
     // should be the shortest.  Rows of different experts are disjoint: the order cannot change a bit.
-    std::vector<int> order;
-    order.reserve(E);
+    std::vector<int> needed;
+    needed.reserve(E);
     for (int e = 0; e < E; ++e)
-        if (count[e] > 0) order.push_back(e);
-    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return count[a] > count[b]; });
+        if (count[e] > 0) needed.push_back(e);
+    std::stable_sort(needed.begin(), needed.end(), [&](int a, int b) { return count[a] > count[b]; });
+    std::vector<int> slotOf(E, -1);
+    for (int s = 0; s < mc; ++s)
+        if (mSlotExpert[s] >= 0) slotOf[mSlotExpert[s]] = s;
+    // Experts still in a slot run first, from there and without a copy; the others follow, most rows first,
+    // through the slots that are not retained.
+    std::vector<int> order;
+    for (const int e : needed)
+        if (slotOf[e] >= 0) order.push_back(e);
+    const int present = (int)order.size(), absent = (int)needed.size() - present;
+    for (const int e : needed)
+        if (slotOf[e] < 0) order.push_back(e);
+    // Retained for the next call: of the experts present, those with most rows, leaving (at most) two slots
+    // for the others to pass through - copy of one under the compute of the other.
+    const int keep = absent == 0 ? present : std::min(present, std::max(0, mc - std::min(2, absent)));
+    // Slots the absent experts pass through, in the order they become free: first those that hold nothing
+    // this call needs, then those of the experts that run from them once more and are then given up (in the
+    // order they run).  Slot numbers break ties, so the choice is deterministic.
+    std::vector<int> streamSlots;
+    for (int s = 0; s < mc; ++s)
+        if (mSlotExpert[s] < 0 || count[mSlotExpert[s]] == 0) streamSlots.push_back(s);
+    for (int k = keep; k < present; ++k) streamSlots.push_back(slotOf[order[k]]);
+    mLastCopies = 0, mLastHits = present;
+    std::vector<int> lastUse(mc, -1);  // position in `order` of the expert that last ran from the slot in this call
     // Whatever happens in the loop, the compute streams forked above are joined back into the caller's
     // stream before returning: an error half way must not leave work that nothing waits for.
     auto queueExperts = [&]() -> Status {
-        int k = 0;
+        int k = 0, turn = 0;
         for (const int e : order) {
-            const int slot = k % mc;
-            char* slotPtr = c.slots + c.slotStride * (size_t)slot;
-            if (k >= mc) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[k - mc], 0));
-            INFMOE_TRY(mSublayer->copyWeights(slotPtr, e, mCopyStream));
-            INFMOE_HIP(hipEventRecord(mCopyDone[k], mCopyStream));
+            int slot = slotOf[e];
             hipStream_t cs = mComputeStreams[k % mComputeStreams.size()];
-            INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
+            if (slot < 0) {
+                slot = streamSlots[turn++ % streamSlots.size()];
+                // the slot's previous expert of this call must be done with it (earlier calls are: the copy
+                // stream was forked from the caller's stream, into which they were joined)
+                if (lastUse[slot] >= 0) INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mComputeDone[lastUse[slot]], 0));
+                mSlotExpert[slot] = -1;  // not valid until the copy has been queued without error
+                INFMOE_TRY(mSublayer->copyWeights(mSlotPool + c.slotStride * (size_t)slot, e, mCopyStream));
+                mSlotExpert[slot] = e;
+                ++mLastCopies;
+                INFMOE_HIP(hipEventRecord(mCopyDone[k], mCopyStream));
+                INFMOE_HIP(hipStreamWaitEvent(cs, mCopyDone[k], 0));
+            }
+            char* slotPtr = mSlotPool + c.slotStride * (size_t)slot;
             // rows of different experts are disjoint, so each expert gets its own stretch of the
             // shared scratch (row stride applied: the public reference omits it at :373,391-392)
             INFMOE_TRY(mSublayer->runInLayer(T, count[e], slotPtr, c.routed + (size_t)offset[e] * d,
                                              c.post + (size_t)offset[e] * d,
                                              c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
             INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
+            lastUse[slot] = k;
             ++k;
         }
         return INFMOE_OK;
@@ -512,6 +563,13 @@ Status MoELayer::lastRouting(int32_t* countHost, int32_t* statsHost) {
     if (statsHost) memcpy(statsHost, tmp.data() + 2 * E + 1, sizeof(int32_t) * 3);
     // the caller has now been told of that call's NaN rows (stats[1]): the next enqueue does not repeat it
     if (tmp[2 * E + 1 + 1] > 0) *static_cast<volatile int32_t*>(mNanFlagHost) = 0;
+    return INFMOE_OK;
+}
+
+Status MoELayer::lastStreaming(int32_t* copies, int32_t* hits) const {
+    if (!mInitialized) return fail(INFMOE_ERR_STATE, "no call before initialize");
+    if (copies) *copies = mLastCopies;
+    if (hits) *hits = mLastHits;
     return INFMOE_OK;
 }
 

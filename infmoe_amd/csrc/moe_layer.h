@@ -44,6 +44,7 @@ class MoELayer {
     Status terminate();                                                        // :203-237
     Status setScoreBias(const float* host);
     Status lastRouting(int32_t* countHost, int32_t* statsHost);
+    Status lastStreaming(int32_t* copies, int32_t* hits) const;
     Status setTiming(int depth);  // 0: off; n: keep the phase marks of the last n calls
     Status lastTiming(float* ms);
     Status timingHistory(float* ms, int maxCalls, int* nCalls);
@@ -80,6 +81,10 @@ class MoELayer {
     int32_t* mNanFlagHost = nullptr;  // in the same allocation: set by the gating kernels, read by the host
     int32_t* mNanFlagDev = nullptr;   // its device address
     int mNanRowsSeen = 0;             // streamed schedule: NaN rows of the call in progress
+    char* mSlotPool = nullptr;        // streamed experts: max_concurrency weight slots, kept between calls
+    std::vector<int> mSlotExpert;     // expert held by each slot, -1 for none
+    uint64_t mSlotVersion = 0;        // sub-layer weights version the slots' contents belong to
+    int mLastCopies = 0, mLastHits = 0;  // of the most recent streamed call
     hipStream_t mCopyStream = nullptr;
     std::vector<hipStream_t> mComputeStreams;
     std::vector<hipEvent_t> mCopyDone, mComputeDone, mJoin;

@@ -77,6 +77,7 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)expert);
     memcpy(slot + off, host, cnt * sizeof(float));
     mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
+    mVersion.fetch_add(1, std::memory_order_acq_rel);
     if (mDeviceWeights != nullptr) {  // already resident: keep the device copy in step (blocking; not a hot path)
         char* dev = static_cast<char*>(mDeviceWeights) + slotStride() * (size_t)expert + off * sizeof(float);
         INFMOE_HIP(hipMemcpy(dev, slot + off, cnt * sizeof(float), hipMemcpyHostToDevice));

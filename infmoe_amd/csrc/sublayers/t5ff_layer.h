@@ -12,6 +12,7 @@
 // product is formed in the GEMM epilogue here, so one is enough).
 #pragma once
 
+#include <atomic>
 #include <vector>
 
 #include "sublayer.h"
@@ -38,6 +39,7 @@ class T5FFLayer : public MoESubLayer {
     void terminate() override;
 
     Status setWeights(int expert, const char* key, const float* host, size_t count) override;
+    uint64_t weightsVersion() const override { return mVersion.load(std::memory_order_acquire); }
     Status makeResident() override;
     const void* residentWeights() const override { return mDeviceWeights; }
     size_t residentStride() const override { return slotStride(); }
@@ -62,6 +64,7 @@ class T5FFLayer : public MoESubLayer {
     float* mHostWeights = nullptr;   // page-locked, E slots of slotStride() bytes
     std::vector<uint8_t> mHave;      // [E][nMatrices+1] which arrays have been provided
     void* mDeviceWeights = nullptr;  // E slots when resident
+    std::atomic<uint64_t> mVersion{0};  // bumped by every setWeights
 };
 
 }  // namespace infmoe

@@ -71,6 +71,12 @@ class Plugin:
         capi.check(self._lib.infmoe_last_routing(self._h, count, stats))
         return np.array(count[:], np.int32), dict(near_ties=stats[0], nan_rows=stats[1], rescored=stats[2])
 
+    def last_streaming(self):
+        """(experts copied host-to-device, experts served from a slot kept from an earlier call) of the last call."""
+        copies, hits = C.c_int32(0), C.c_int32(0)
+        capi.check(self._lib.infmoe_last_streaming(self._h, C.byref(copies), C.byref(hits)))
+        return copies.value, hits.value
+
     PHASES = ("gating", "count_sort", "scatter", "expert_norm", "expert_gemm1", "expert_gemm2", "gather")
 
     def set_timing(self, enable) -> None:

@@ -132,6 +132,64 @@ def test_output_is_bit_identical_for_every_max_concurrency(torch_cuda, variant):
         np.testing.assert_array_equal(o, outs[0])
 
 
+@pytest.mark.parametrize("mc", [1, 2, 3, 4, 6])
+def test_slots_keep_experts_between_calls(torch_cuda, mc):
+    """Streamed experts stay in their slots: an expert needed again is not copied again, whatever mix of
+    experts the calls need, and the output is that of the resident layer bit for bit on every call."""
+    torch = torch_cuda
+    shape, E, d, h = (2, 80), 8, 64, 192
+    B, S = shape
+    resident, x, c, g, ws = make_layer(shape, E, d, h, E, "cpm_2", seed=83)
+    streamed, *_ = make_layer(shape, E, d, h, mc, "cpm_2", seed=83)
+    rng = np.random.default_rng(1)
+    # inputs that need different subsets of the experts: all of them, then tokens of three experts only, ...
+    sel = O.gate(x, c, "cpm_2", g)[0]
+    inputs = [x, x[np.isin(sel, [0, 1, 2])][:B * S // 4], x[np.isin(sel, [1, 2, 5, 6])][:B * S // 4], x, x]
+    history = []
+    for i, xi in enumerate(inputs):
+        xi = np.ascontiguousarray(xi)
+        dx = dev(torch, xi.reshape(1, -1, d))
+        want = resident.forward(dx)
+        got = streamed.forward(dx)
+        assert torch.equal(got, want), f"call {i} differs from the resident layer"
+        count, _ = streamed.last_routing()
+        needed = set(np.flatnonzero(count > 0).tolist())
+        copies, hits = streamed.last_streaming()
+        assert copies + hits == len(needed) and 0 <= hits <= mc
+        history.append((needed, copies, hits))
+    assert len(history[0][0]) == E and history[0][1:] == (E, 0)      # first call: every expert copied
+    assert history[1][0] == {0, 1, 2} and history[2][0] == {1, 2, 5, 6}
+    if mc >= 3:
+        assert history[2][2] >= 2          # experts 1 and 2 ran in call 1 and were still there
+    if mc >= 6:
+        assert history[2][1] <= 2          # ... and with room to spare nothing else was displaced for them
+    # calls 3 and 4 need all eight experts: after call 3 every slot holds one of them, so call 4 copies the rest only
+    assert history[4][2] == mc and history[4][1] == E - mc
+    assert_close(got.cpu().numpy().reshape(-1, d), O.moe_layer(x, c, "cpm_2", ws, layernorm_weight=g)["out"], what="last call")
+    assert resident.last_streaming() == (0, 0)
+    resident.terminate()
+    streamed.terminate()
+
+
+def test_new_weights_empty_the_slots(torch_cuda):
+    torch = torch_cuda
+    shape, E, d, h = (2, 40), 4, 64, 128
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, 4 - 1, "default", seed=89)
+    dx = dev(torch, x.reshape(2, 40, d))
+    plugin.forward(dx)
+    plugin.forward(dx)
+    copies, hits = plugin.last_streaming()
+    assert hits > 0
+    ws[1] = O.draw_expert(90, 1, d, h)
+    for k, v in ws[1].items():
+        plugin.set_expert_weights(1, k, v)
+    y = plugin.forward(dx).cpu().numpy().reshape(-1, d)
+    copies, hits = plugin.last_streaming()
+    assert hits == 0 and copies > 0
+    assert_close(y, O.moe_layer(x, c, "default", ws)["out"], what="after new weights")
+    plugin.terminate()
+
+
 @pytest.mark.parametrize("d,h", [(40, 72), (30, 50)])  # multiples of 4 but not of 32; not even of 4
 @pytest.mark.parametrize("variant,ffn", [("cpm_2", "relu"), ("base_layer", "gated_gelu")])
 @pytest.mark.parametrize("mc", [2, 4])

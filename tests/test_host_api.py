@@ -130,15 +130,16 @@ def test_workspace_size_accounting():
     slot = 4 * (d + 2 * d * h)
     streamed = workspace(GOOD, (2, 50, d))
     resident = workspace({**GOOD, "max_concurrency": E}, (2, 50, d))
-    # streamed experts add max_concurrency slots (each rounded up to 256 bytes); resident ones live in
-    # plugin-owned memory (the reference always carves the slots from the workspace, MoELayerPlugin.cc:243-264)
-    assert streamed - resident == 2 * ((slot + 255) // 256 * 256)
+    # the weight slots of streamed experts and the resident experts are both memory of the layer (the reference
+    # carves the slots from the workspace, MoELayerPlugin.cc:243-264; slots that keep experts between calls
+    # cannot live in memory the caller may hand to others between calls)
+    assert streamed == resident and slot > 0
     T = 100
     floor = 4 * (T * (d + h) + 3 * T + 2 * T + 2 * T * d)  # sub-layer scratch, sel/pos/rowExpert, coeffs, routed+post
     assert floor <= resident <= floor + 64 * 256
     assert workspace({**GOOD, "max_concurrency": E}, (2, 100, d)) > resident
     gated = workspace({**GOOD, "ffn_kind": "gated_gelu"}, (2, 50, d))
-    assert gated - streamed == 2 * ((4 * (d + 3 * d * h) + 255) // 256 * 256) - 2 * ((slot + 255) // 256 * 256)
+    assert gated == streamed  # one hidden buffer in either form: the gelu*mul product is formed in the GEMM epilogue
     ident = workspace({**GOOD, "expert_sublayer_type": "Identity"}, (2, 50, d))
     assert ident < resident
 
