@@ -41,6 +41,9 @@ CONFIGS = {
     "c3": dict(variant="cpm_2", E=32, d=4096, h=10240, mc=2, shape=(8, 512), zipf=False),
     "c4": dict(variant="base_layer", E=64, d=2048, h=8192, mc=64, shape=(16, 1024), zipf=True),
     "c5": dict(variant="cpm_2", E=32, d=4096, h=10240, mc=32, shape=(64, 1), zipf=False),
+    # the reference's own example (python/examples/stacked_moe.py:23-27): three stacked layers that share one
+    # sub-layer, 80 x 512 tokens, experts streamed through four slots
+    "ex": dict(variant="cpm_2", E=20, d=4096, h=16384, mc=4, shape=(80, 512), zipf=False, layers=3),
 }
 
 
@@ -132,7 +135,7 @@ def cpu_baseline(cfg, x, cent, gamma, slots, bias, sample_tokens):
                       f"oracle/moe_cpu.c (FP32, OpenMP, AVX2), {dt:.2f} s"}
 
 
-def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False):
+def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None):
     """W untimed steps, then K timed ones between two events on the layer's stream, with the library's phase
     marks (HIP events on the same stream) kept for exactly those K steps."""
     n_mat = 3 if gated else 2  # weight matrices of an expert
@@ -144,8 +147,15 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False):
     y = torch.empty_like(x)
     stream = torch.cuda.current_stream().cuda_stream
 
-    def step():
-        plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
+    if stack:  # layers that share the sub-layer, each fed with its predecessor's output; one workspace for all
+        bufs = [x, y, torch.empty_like(x)]
+
+        def step():
+            for i, layer in enumerate(stack):
+                layer.enqueue(dims, bufs[i % 3].data_ptr(), bufs[(i + 1) % 3].data_ptr(), ws.data_ptr(), stream)
+    else:
+        def step():
+            plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
 
     plugin.set_timing(steps)  # HIP events at the phase boundaries, kept for every step of the timed region
     for _ in range(warmup):
@@ -175,12 +185,14 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False):
     gemm_ms = (phases["expert_gemm1"] + phases["expert_gemm2"]) / n_mat
     launches = ("two launches per step: wi_0 and wi_1 with gelu*mul, wo with residual; figures per weight matrix"
                 if gated else "two launches per step: wi with ReLU, wo with residual")
-    if not resident:
-        # streamed experts: the host link bounds the call, not HBM and not the matrix core
-        bytes_per_call = active * 4.0 * (d + n_mat * d * h)
+    copies = plugin.last_streaming()[0] if not resident else 0
+    if not resident and copies > 0:
+        # streamed experts: the host link bounds the call, not HBM and not the matrix core (experts still in a
+        # slot from the call before are not copied again)
+        bytes_per_call = copies * 4.0 * (d + n_mat * d * h)
         roofline = {"bound": "pcie", "achieved": round(bytes_per_call / (phases["expert_gemm1"] * 1e-3) / 1e9, 2),
                     "peak": PCIE_PEAK_GBS, "unit": "GB/s", "traffic": None,
-                    "kernel": "host-to-device expert copies overlapped with expert kernels",
+                    "kernel": f"host-to-device copies of {copies} of {active} active experts overlapped with expert kernels",
                     "note": "bounded by the host link (PCIe Gen5 x16, 64 GB/s per direction): achieved = streamed weight "
                             "bytes / expert-loop time"}
     elif few_rows:
@@ -242,6 +254,7 @@ def main():
     ap.add_argument("--sweep-tokens", default="",
                     help="comma-separated token counts: after the workload proper, the same layer is timed on that many "
                          "tokens of the batch each (e.g. 256,512,1024,2048 with c2: 8 to 64 rows per expert)")
+    ap.add_argument("--mc", type=int, default=0, help="override the workload's max_concurrency")
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: do not also measure the decode shape (c5) and the skewed one (c4)")
     ap.add_argument("--replicate-weights", action="store_true",
@@ -258,6 +271,8 @@ def main():
     capi.load()  # fails loudly when the HIP library has not been built
 
     cfg = dict(CONFIGS[args.config], ffn=args.ffn)
+    if args.mc > 0:
+        cfg["mc"] = args.mc
     gated = args.ffn == "gated_gelu"
     if gated:
         args.no_cpu = True
@@ -268,7 +283,15 @@ def main():
     torch.cuda.set_device(0)
     plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=not args.no_cpu,
                                                       replicate=args.replicate_weights)
-    m = measure(torch, plugin, cfg, args.config, x, args.steps, args.warmup, gated)
+    stack = None
+    if cfg.get("layers", 1) > 1:  # clones share the sub-layer and so the host copy of the weights
+        stack = [plugin]
+        for _ in range(cfg["layers"] - 1):
+            twin = plugin.clone()
+            twin.configure([B, S, d])
+            twin.initialize()
+            stack.append(twin)
+    m = measure(torch, plugin, cfg, args.config, x, args.steps, args.warmup, gated, stack=stack)
     count, stats, active, resident = m["count"], m["stats"], m["active"], m["resident"]
     ms_per_step, wall_ms, phases, last = m["ms_per_step"], m["wall_ms"], m["phases"], m["last"]
     roofline, phase_rates = m["roofline"], m["phase_rates"]
@@ -297,6 +320,12 @@ def main():
         "host_ms_per_step": round(wall_ms, 4),
         "routing": stats,
     }
+    if stack:
+        out["config"]["stacked_layers"] = len(stack)
+        out["value"] = round(T / (ms_per_step * 1e-3), 1)  # tokens through the whole stack per second
+    if not resident:
+        copies, hits = plugin.last_streaming()
+        out["streaming_last_call"] = {"experts_copied": copies, "experts_found_in_slots": hits}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, x, cent, gamma, slots, bias, min(args.cpu_sample, T))
     # Further workloads of the same run (the headline `value` above is untouched by them):

@@ -76,6 +76,14 @@ struct GroupedRun {
     const RowTile* tiles = nullptr;     /* device: scheduled row tiles */
     const int32_t* sched = nullptr;     /* device, 16 ints: [0] number of tiles, [1 + x] first tile of die x's share */
     int32_t maxTiles = 0;               /* upper bound of [0], known on the host */
+    /* Where the experts' weights are.  Null: the sub-layer's own resident copy (makeResident).  Else the base
+     * of weight slots of `weightStride` bytes each, expert e in slot expertSlot[e] (device [E]; an entry is
+     * only meaningful for an expert with rows): the layer's slots when every expert of a call with streamed
+     * experts is already in one. */
+    const void* weights = nullptr;
+    size_t weightStride = 0;
+    const int32_t* expertSlot = nullptr;
+    const int32_t* expertSlotHost = nullptr; /* the same table in host memory */
     hipStream_t stream = nullptr;
     hipEvent_t afterNorm = nullptr, afterGemm1 = nullptr; /* optional phase marks to record on `stream` */
 };
@@ -141,6 +149,8 @@ class MoESubLayer {
     /* All experts of one call, weights resident.  The default copies count / offset to the host (one wait
      * on the stream) and calls runInLayer once per expert with rows, in ascending index, on g.stream. */
     virtual Status runGrouped(const GroupedRun& g);
+    /* Whether runGrouped honours g.weights / g.expertSlot (the default one does). */
+    virtual bool groupedFromSlots() const { return true; }
     int expertCount() const { return mExpertCount; }
 
    private:

@@ -19,7 +19,9 @@ __global__ void expert_gemm_generic_kernel(GemmProblem p, int rows, size_t weigh
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)rows * p.N) return;
     const int row = idx / p.N, col = idx % p.N;
-    const size_t w0 = row_expert ? (size_t)row_expert[row] * weight_stride : 0;
+    int owner = row_expert ? row_expert[row] : 0;
+    if (row_expert && p.expert_slot) owner = p.expert_slot[owner];
+    const size_t w0 = (size_t)owner * weight_stride;
     const float* a = p.A + (size_t)row * p.K;
     const float* b0 = p.B + w0 + (size_t)col * p.K;
     float s0 = 0.f, s1 = 0.f;

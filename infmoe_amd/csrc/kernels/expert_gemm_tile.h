@@ -417,8 +417,9 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProbl
     if (slot >= share * n_col_tiles) return;
     const RowTile rt = tiles[first + slot / n_col_tiles];
     const int n0 = (slot % n_col_tiles) * BN;
-    const float* B0 = p.B + (size_t)rt.expert * weight_stride;
-    const float* B1 = GATED ? p.B1 + (size_t)rt.expert * weight_stride : nullptr;
+    const int owner = p.expert_slot ? p.expert_slot[rt.expert] : rt.expert;
+    const float* B0 = p.B + (size_t)owner * weight_stride;
+    const float* B1 = GATED ? p.B1 + (size_t)owner * weight_stride : nullptr;
     gemm_dispatch<BN, GATED>(p.A + (size_t)rt.row0 * p.K, p.R ? p.R + (size_t)rt.row0 * p.N : nullptr,
                              p.C + (size_t)rt.row0 * p.N, rt.rows, B0, B1, n0, p.N, p.K, p.epilogue, smem,
                              GATED ? kGemmTileRowsGated : kGemmTileRows);

@@ -178,8 +178,9 @@ __global__ __launch_bounds__(kThreads, GATED ? 2 : 3) void expert_skinny_kernel(
         const int e = blockIdx.y;
         rows = count[e];
         row0 = offset[e];
-        B0 += (size_t)e * weight_stride;
-        if (GATED) B1 += (size_t)e * weight_stride;
+        const int owner = p.expert_slot ? p.expert_slot[e] : e;
+        B0 += (size_t)owner * weight_stride;
+        if (GATED) B1 += (size_t)owner * weight_stride;
     }
     if (rows <= 0 || rows > kSkinnyMaxRows) return;
     const float* A = p.A + (size_t)row0 * p.K;

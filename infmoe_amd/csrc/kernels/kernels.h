@@ -123,9 +123,11 @@ hipError_t launch_mix_gather(int T, int d, const int* pos, const float* routed, 
                              const float* routed_coeff, float* out, hipStream_t stream);
 
 // ---- row norm (replaces layernorm_gpu, plugin/cuda/ops/layernorm.cu:176-188)
-// gamma of row r is gamma_base + row_expert[r] * gamma_stride (row_expert null -> gamma_base).
+// gamma of row r is gamma_base + slot(row_expert[r]) * gamma_stride (row_expert null -> gamma_base), where
+// slot(e) = expert_slot[e], or e when expert_slot is null.
 hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const float* gamma_base,
-                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream);
+                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream,
+                           const int* expert_slot = nullptr);
 
 // ---- expert GEMMs (replace the three cublasSgemm_v2 calls, fused_gelu_dot_gpu and the D2D
 //      residual copy of plugin/sublayers/T5FFLayer.cc:112-138)
@@ -142,6 +144,9 @@ struct GemmProblem {
     float* C;          // [rows][N]
     int N, K;
     int epilogue;
+    // grouped launches only: null, or [E] where expert e's weights are at B + expert_slot[e] * weight_stride
+    // instead of B + e * weight_stride (experts held in slots in whatever order they arrived)
+    const int* expert_slot;
 };
 // One expert, `rows` known on the host, cut into row tiles of at most `tile_rows` rows (a multiple of
 // 16 no larger than gemm_tile_rows(p.epilogue); both launches of a sub-layer pass the same value so

@@ -30,13 +30,15 @@ template <bool VEC, int RV>
 __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                             int rows, int d, const float* __restrict__ gamma_base,
                                                             size_t gamma_stride, const int* __restrict__ row_expert,
-                                                            int norm_kind) {
+                                                            int norm_kind, const int* __restrict__ expert_slot) {
     const int lane = threadIdx.x & 63;
     const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (r >= rows) return;
     const float* x = in + (size_t)r * d;
     float* y = out + (size_t)r * d;
-    const float* g = gamma_base + (row_expert ? (size_t)row_expert[r] * gamma_stride : 0);
+    int owner = row_expert ? row_expert[r] : 0;
+    if (row_expert && expert_slot) owner = expert_slot[owner];
+    const float* g = gamma_base + (size_t)owner * gamma_stride;
     const float inv_d = 1.0f / (float)d;
 
     if (VEC && d <= 64 * 4 * RV) {
@@ -89,7 +91,8 @@ __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ 
 }  // namespace
 
 hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const float* gamma_base,
-                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream) {
+                           size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream,
+                           const int* expert_slot) {
     if (rows <= 0) return hipSuccess;
     const dim3 grid((rows + kThreads / 64 - 1) / (kThreads / 64));
     const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in) |
@@ -97,7 +100,7 @@ hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const f
                          (gamma_stride % 4 == 0);
 #define INFMOE_NORM(V, RV)                                                                                        \
     row_norm_kernel<V, RV><<<grid, kThreads, 0, stream>>>(out, in, rows, d, gamma_base, gamma_stride, row_expert, \
-                                                          norm_kind)
+                                                          norm_kind, expert_slot)
     if (d % 4 == 0 && aligned) {
         if (d <= 2048) INFMOE_NORM(true, 8);
         else if (d <= 4096) INFMOE_NORM(true, 16);

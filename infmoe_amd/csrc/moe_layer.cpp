@@ -250,6 +250,9 @@ Status MoELayer::initializeSteps() {
         INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mSlotPool), stride * (size_t)mParams.maxConcurrency));
         mSlotExpert.assign(mParams.maxConcurrency, -1);
         mSlotVersion = mSublayer->weightsVersion();
+        INFMOE_HIP(hipMalloc(reinterpret_cast<void**>(&mSlotTableGpu), sizeof(int32_t) * E));
+        INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mSlotTableHost), sizeof(int32_t) * E, hipHostMallocDefault));
+        mSlotTableSent.clear();
         INFMOE_HIP(hipStreamCreateWithFlags(&mCopyStream, hipStreamNonBlocking));
         mComputeStreams.resize(std::min(mParams.maxConcurrency, 4));
         for (auto& s : mComputeStreams) INFMOE_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
@@ -284,6 +287,10 @@ Status MoELayer::terminate() {
     if (mSlotPool) (void)hipFree(mSlotPool);
     mSlotPool = nullptr;
     mSlotExpert.clear();
+    if (mSlotTableGpu) (void)hipFree(mSlotTableGpu);
+    if (mSlotTableHost) (void)hipHostFree(mSlotTableHost);
+    mSlotTableGpu = mSlotTableHost = nullptr;
+    mSlotTableSent.clear();
     for (auto s : mComputeStreams) (void)hipStreamDestroy(s);
     mComputeStreams.clear();
     for (auto* v : {&mCopyDone, &mComputeDone, &mJoin}) {
@@ -344,35 +351,35 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
                                 /*zero_stats=*/true, mNanFlagDev));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
+    // (the row tiles of the grouped expert launch are made on either schedule: streamed experts that are all
+    // still in their slots run from one set of launches too)
     const bool grouped = resident();
-    const int skinnyMax = grouped ? mSublayer->skinnyMaxRows(T) : 0;
-    INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, grouped ? c.tiles : nullptr,
-                                   grouped ? c.sched : nullptr, mSublayer->rowTileHeight(), skinnyMax, c.rowExpert, stream));
+    const int skinnyMax = mSublayer->skinnyMaxRows(T);
+    INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, c.tiles, c.sched,
+                                   mSublayer->rowTileHeight(), skinnyMax, c.rowExpert, stream));
     INFMOE_TRY(mark(2));
     INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream));  // experts see the raw input (:354)
     INFMOE_HIP(hipEventRecord(mRoutingDone, stream));
     INFMOE_TRY(mark(3));
 
     // 4. experts                                                   plugin/MoELayerPlugin.cc:360-402
+    GroupedRun g;
+    g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
+    g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
+    g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
+    if (skinnyMax > 0) {
+        // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
+        // of them, each with one tile more than its rows fill.  A decode call then launches a small
+        // grid (or none) for the matrix-core kernel instead of one sized for E experts.
+        const int tall = T / (skinnyMax + 1);
+        g.maxTiles = std::min(c.maxTiles, tall + T / mSublayer->rowTileHeight());
+    }
+    if (timed) g.afterNorm = marks[4], g.afterGemm1 = marks[5];
     if (grouped) {
-        GroupedRun g;
-        g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
-        g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
-        g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
-        if (skinnyMax > 0) {
-            // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
-            // of them, each with one tile more than its rows fill.  A decode call then launches a small
-            // grid (or none) for the matrix-core kernel instead of one sized for E experts.
-            const int tall = T / (skinnyMax + 1);
-            g.maxTiles = std::min(c.maxTiles, tall + T / mSublayer->rowTileHeight());
-        }
-        if (timed) g.afterNorm = marks[4], g.afterGemm1 = marks[5];
         INFMOE_TRY(mSublayer->runGrouped(g));
     } else {
-        INFMOE_TRY(mark(4));
         mNanRowsSeen = 0;
-        INFMOE_TRY(runStreamed(T, c, stream));
-        INFMOE_TRY(mark(5));
+        INFMOE_TRY(runStreamed(T, c, stream, g));
     }
     INFMOE_TRY(mark(6));
 
@@ -456,7 +463,7 @@ Status MoELayer::lastTiming(float* ms) {
 // through (copy of one under the compute of the other); the rest are copied, most rows first.  A change of
 // any expert's weights (infmoe_set_expert_weights) empties the slots.  Which expert sits where has no
 // influence on the arithmetic: the output is the same bit for bit.
-Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
+Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedRun& g) {
     const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
     const size_t routingInts = (size_t)2 * E + 1 + 4;
     INFMOE_HIP(hipMemcpyAsync(mRoutingHost, mRoutingGpu, sizeof(int32_t) * routingInts, hipMemcpyDeviceToHost, stream));
@@ -468,9 +475,6 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
     // reports them when everything is queued (this schedule knows of them now; the resident one later)
     mNanRowsSeen = stats[1];
 
-    INFMOE_HIP(hipEventRecord(mFork, stream));
-    INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
-    for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
     if (mSublayer->weightsVersion() != mSlotVersion) {  // some expert's weights changed: nothing cached is valid
         std::fill(mSlotExpert.begin(), mSlotExpert.end(), -1);
         mSlotVersion = mSublayer->weightsVersion();
@@ -506,6 +510,21 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
         if (mSlotExpert[s] < 0 || count[mSlotExpert[s]] == 0) streamSlots.push_back(s);
     for (int k = keep; k < present; ++k) streamSlots.push_back(slotOf[order[k]]);
     mLastCopies = 0, mLastHits = present;
+    if (absent == 0 && mSublayer->groupedFromSlots()) {
+        // Every expert of the call is in a slot already: one set of launches over all of them, as when the
+        // experts are resident, with a table that says which slot holds which expert.
+        if (slotOf != mSlotTableSent) {
+            memcpy(mSlotTableHost, slotOf.data(), sizeof(int32_t) * E);
+            INFMOE_HIP(hipMemcpyAsync(mSlotTableGpu, mSlotTableHost, sizeof(int32_t) * E, hipMemcpyHostToDevice, stream));
+            mSlotTableSent = slotOf;
+        }
+        g.weights = mSlotPool, g.weightStride = c.slotStride, g.expertSlot = mSlotTableGpu, g.expertSlotHost = slotOf.data();
+        return mSublayer->runGrouped(g);
+    }
+    if (g.afterNorm) INFMOE_HIP(hipEventRecord(g.afterNorm, stream));  // the whole expert loop is reported as one phase
+    INFMOE_HIP(hipEventRecord(mFork, stream));
+    INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
+    for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
     std::vector<int> lastUse(mc, -1);  // position in `order` of the expert that last ran from the slot in this call
     // Whatever happens in the loop, the compute streams forked above are joined back into the caller's
     // stream before returning: an error half way must not leave work that nothing waits for.
@@ -549,6 +568,7 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream) {
         INFMOE_HIP(hipEventRecord(mJoin[i], mComputeStreams[i]));
         INFMOE_HIP(hipStreamWaitEvent(stream, mJoin[i], 0));
     }
+    if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, stream));
     if (queued != INFMOE_OK) last_error_slot() = why;
     return queued;
 }

@@ -62,7 +62,7 @@ class MoELayer {
     Status carve(int T, void* workspace, Carve* c) const;
     bool resident() const;
     Status checkDims(const int32_t* dims, int32_t nbDims, int* tokens) const;
-    Status runStreamed(int T, const Carve& c, hipStream_t stream);
+    Status runStreamed(int T, const Carve& c, hipStream_t stream, GroupedRun& g);
     Status initializeSteps();
 
     MoEParams mParams;
@@ -83,6 +83,9 @@ class MoELayer {
     int mNanRowsSeen = 0;             // streamed schedule: NaN rows of the call in progress
     char* mSlotPool = nullptr;        // streamed experts: max_concurrency weight slots, kept between calls
     std::vector<int> mSlotExpert;     // expert held by each slot, -1 for none
+    int32_t* mSlotTableGpu = nullptr;   // [E] slot of every expert, for launches over all experts from the slots
+    int32_t* mSlotTableHost = nullptr;  // page-locked staging of the same
+    std::vector<int> mSlotTableSent;    // what the device copy holds
     uint64_t mSlotVersion = 0;        // sub-layer weights version the slots' contents belong to
     int mLastCopies = 0, mLastHits = 0;  // of the most recent streamed call
     hipStream_t mCopyStream = nullptr;

@@ -41,11 +41,15 @@ Status MoESubLayer::runGrouped(const GroupedRun& g) {
     INFMOE_HIP(hipStreamSynchronize(g.stream));
     const int32_t* count = host.data();
     const int32_t* offset = host.data() + E;
-    const char* weights = static_cast<const char*>(residentWeights());
+    const bool slots = g.weights != nullptr;
+    const char* weights = static_cast<const char*>(slots ? g.weights : residentWeights());
+    const size_t stride = slots ? g.weightStride : residentStride();
+    if (slots && g.expertSlotHost == nullptr) return fail(INFMOE_ERR_INVALID_ARGUMENT, "grouped run from slots without the slot table");
     const size_t d = (size_t)mEmbeddingSize;
     for (int e = 0; e < E; ++e) {  // ascending, empties skipped (plugin/MoELayerPlugin.cc:361-363,383-384)
         if (count[e] <= 0) continue;
-        INFMOE_TRY(runInLayer(g.tokenCount, count[e], weights ? weights + residentStride() * (size_t)e : nullptr,
+        const size_t owner = slots ? (size_t)g.expertSlotHost[e] : (size_t)e;
+        INFMOE_TRY(runInLayer(g.tokenCount, count[e], weights ? weights + stride * owner : nullptr,
                               g.input + (size_t)offset[e] * d, g.output + (size_t)offset[e] * d,
                               static_cast<char*>(g.workspace) + workspaceOffset(offset[e]), g.stream));
     }

@@ -216,18 +216,21 @@ Status T5FFLayer::runInLayer(int32_t layerTokens, int32_t tokenCount, const void
 }
 
 Status T5FFLayer::runGrouped(const GroupedRun& g) {
-    if (mDeviceWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: runGrouped needs resident weights");
+    if (mDeviceWeights == nullptr && g.weights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: runGrouped needs resident weights");
     const int T = g.tokenCount, d = mEmbeddingSize, h = mHiddenSize;
-    const size_t dh = (size_t)d * h, stride = slotStride() / sizeof(float);
-    const float* w = static_cast<const float*>(mDeviceWeights);
+    const size_t dh = (size_t)d * h, stride = (g.weights ? g.weightStride : slotStride()) / sizeof(float);
+    const float* w = static_cast<const float*>(g.weights ? g.weights : mDeviceWeights);
+    const int* slot = g.weights ? g.expertSlot : nullptr;
     float* ln = static_cast<float*>(g.workspace);
     float* hid = ln + (size_t)T * d;
-    INFMOE_HIP(launch_row_norm(ln, g.input, T, d, w, stride, g.rowExpert, mNormKind, g.stream));
+    INFMOE_HIP(launch_row_norm(ln, g.input, T, d, w, stride, g.rowExpert, mNormKind, g.stream, slot));
     GemmProblem g1{};
+    g1.expert_slot = slot;
     g1.A = ln, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
     g1.B1 = mFfnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
     g1.epilogue = mFfnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
     GemmProblem g2{};
+    g2.expert_slot = slot;
     g2.A = hid, g2.B = w + d + (mFfnKind == FFN_GATED_GELU ? 2 : 1) * dh, g2.R = g.input, g2.C = g.output, g2.N = d, g2.K = h;
     g2.epilogue = EPI_RESIDUAL;
     const bool skinny = skinnyMaxRows(T) > 0;
