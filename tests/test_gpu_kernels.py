@@ -113,6 +113,33 @@ def test_gate_near_tie_is_rescored_in_float64(lib, torch_cuda):
     assert stats[0] == exempt
 
 
+@pytest.mark.parametrize("T,d", [(300, 8192), (1536, 8192), (2048, 16384)])  # one-kernel / sliced form; slab form
+@pytest.mark.parametrize("norm", ["none", "rms"])
+def test_gate_adversarial_same_sign_near_ties(lib, torch_cuda, T, d, norm):
+    """The case in which FP32 accumulation is worst: every term of every dot product has the same sign, the
+    rows are long, and the experts' scores lie a few 1e-6 relative apart (above the 1e-6 exemption, so the
+    assignment has to be the float64 one).  The re-scoring threshold (8 eps times the Cauchy-Schwarz bound of a
+    score, at least 4e-6 of the best score) is an empirical choice, not a worst-case bound of a length-d FP32
+    sum; this pins it where it is most at risk."""
+    torch = torch_cuda
+    E = 16
+    rng = np.random.default_rng(d + T)
+    x = (np.abs(rng.standard_normal((T, d))) + 0.5).astype(np.float32)
+    c0 = (np.abs(rng.standard_normal(d)) + 0.1) / np.sqrt(d)
+    order = rng.permutation(E)  # the best expert is not the last index
+    c = np.stack([c0 * (1.0 + 2.5e-6 * order[e]) for e in range(E)]).astype(np.float32)
+    g = (1.0 + 0.1 * np.abs(rng.standard_normal(d))).astype(np.float32)
+    sel, coeff, stats = run_gate(lib, torch, x, c, g if norm != "none" else None, norm)
+    xa = O.layernorm(x, g, norm) if norm != "none" else x.astype(np.float64)
+    aff = O.score(xa, c)
+    gap = O.top2_relative_gap(aff)
+    assert (gap < 1e-5).all() and (gap > 1e-6).mean() > 0.9  # near ties everywhere, nearly none of them exempt
+    exempt = check_assignment(sel, aff)
+    assert stats[0] == exempt
+    assert stats[2] >= T // 2  # FP32 could not be trusted with most of them: the float64 path decided
+    assert_close(coeff, aff[np.arange(T), sel], what="coeff")
+
+
 # ------------------------------------------------------------------ count / sort
 @pytest.mark.parametrize("T,E,mode", [
     (1, 1, "rand"), (1, 4, "rand"), (32, 4, "rand"), (1023, 7, "rand"), (1024, 32, "rand"), (1025, 32, "rand"),
