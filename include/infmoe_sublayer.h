@@ -73,6 +73,7 @@ struct GroupedRun {
     const int32_t* count = nullptr;     /* device [E]: rows of every expert */
     const int32_t* offset = nullptr;    /* device [E+1]: first routed row of every expert */
     const int32_t* rowExpert = nullptr; /* device [T]: expert of every routed row */
+    const float* rowStats = nullptr;    /* device [T][2]: (mean, reciprocal deviation) of every routed row, when rowStatsKind() asks for them */
     const RowTile* tiles = nullptr;     /* device: scheduled row tiles */
     const int32_t* sched = nullptr;     /* device, 16 ints: [0] number of tiles, [1 + x] first tile of die x's share */
     int32_t maxTiles = 0;               /* upper bound of [0], known on the host */
@@ -123,9 +124,14 @@ class MoESubLayer {
      * that picks between kernels by the shape of the whole call does it here, from its arguments only, so
      * that layers that share the sub-layer (clones) cannot influence each other. */
     virtual Status runInLayer(int32_t /*layerTokens*/, int32_t tokenCount, const void* weights, const void* input,
-                              void* output, void* workspace, hipStream_t stream) {
+                              void* output, void* workspace, hipStream_t stream, const float* /*rowStats*/ = nullptr) {
         return run(tokenCount, weights, input, output, workspace, stream);
     }
+    /* Row statistics the layer's scatter computes while it copies the routed rows, for experts that start with
+     * a row norm: INFMOE_NORM_NONE (none), INFMOE_NORM_RMS: (0, rsqrt(mean(x^2) + 1e-6)), INFMOE_NORM_CENTERED:
+     * (mean, rsqrt(biased variance + 1e-6)).  They arrive as GroupedRun::rowStats and as runInLayer's last
+     * argument (there for the expert's own rows). */
+    virtual int rowStatsKind() const { return INFMOE_NORM_NONE; }
     /* Where, inside a scratch of workspaceSize(T) bytes, the expert whose rows start at routed row
      * `firstRow` may work without touching another expert's stretch. */
     virtual size_t workspaceOffset(int32_t /*firstRow*/) { return 0; }

@@ -20,11 +20,13 @@ LIB_PATH = os.path.join(LIB_DIR, "libinfmoe.so")
 SOURCES = [
     "kernels/dispatch.hip",
     "kernels/norm.hip",
-    # the four instantiations of the matrix-core expert kernel first: they take longest
-    "kernels/expert_gemm_grouped.hip",
-    "kernels/expert_gemm_one.hip",
+    # the six instantiations of the matrix-core expert kernel first: they take longest
     "kernels/expert_gemm_grouped_gated.hip",
     "kernels/expert_gemm_one_gated.hip",
+    "kernels/expert_gemm_grouped_relu.hip",
+    "kernels/expert_gemm_one_relu.hip",
+    "kernels/expert_gemm_grouped.hip",
+    "kernels/expert_gemm_one.hip",
     "kernels/expert_gemm.hip",
     "kernels/gating.hip",
     "kernels/gating_slab.hip",

@@ -369,7 +369,7 @@ int32_t infmoe_t5ff_run(int32_t rows, int32_t d, int32_t h, int32_t norm_kind, i
         INFMOE_NEED(ffn_kind == FFN_RELU || ffn_kind == FFN_GATED_GELU, "t5ff_run: bad ffn_kind");
         INFMOE_NEED(rows == 0 || (weights && in && out && workspace), "t5ff_run: null pointer");
         return T5FFLayer::runOne(rows, rows, 1, d, h, norm_kind, ffn_kind, weights, in, out, workspace,
-                                 static_cast<hipStream_t>(hip_stream));
+                                 static_cast<hipStream_t>(hip_stream), /*folded=*/false, nullptr);
     });
 }
 

@@ -272,6 +272,99 @@ __global__ __launch_bounds__(kThreads) void scatter_kernel(int T, int d, const f
     if (lane == 0 && coeff != nullptr && routed_coeff != nullptr) routed_coeff[r] = coeff[t];
 }
 
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// The scatter with the row statistics of the experts' norm computed on the way (COPY), or the statistics alone
+// of rows where they lie (pos == nullptr, no copy): stats[r] = (mu, rstd) of routed row r, as the first expert
+// product wants them (the norm itself is folded into that product).  rms: mu = 0, rstd = rsqrt(mean(x^2) +
+// eps).  centered: the mean, then a second sweep over the row (it has just been read: it comes from cache)
+// for the variance about the mean - the exact two-pass form (plugin/cuda/ops/layernorm.cu:30-130 merges
+// Welford partials instead).  Both launches run this code, so the numbers agree bit for bit.
+template <bool VEC, bool COPY>
+__global__ __launch_bounds__(kThreads) void scatter_stats_kernel(int T, int d, const float* __restrict__ x,
+                                                                 const float* __restrict__ coeff,
+                                                                 const int* __restrict__ pos,
+                                                                 float* __restrict__ routed,
+                                                                 float* __restrict__ routed_coeff,
+                                                                 float* __restrict__ stats, int norm_kind) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (r >= T) return;
+    const int t = pos != nullptr ? pos[r] : r;
+    const float* src = x + (size_t)t * d;
+    float* dst = COPY ? routed + (size_t)r * d : nullptr;
+    float s1 = 0.f, s2 = 0.f;
+    if (VEC) {
+        const int n4 = d >> 2;
+        const v4f* s = reinterpret_cast<const v4f*>(src);
+        v4f* o = reinterpret_cast<v4f*>(dst);
+        float p1[4] = {0.f, 0.f, 0.f, 0.f}, p2[4] = {0.f, 0.f, 0.f, 0.f};
+        auto take = [&](const v4f& v, int q) {
+            p1[q] += (v.x + v.y) + (v.z + v.w);
+            p2[q] += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        };
+        int k = lane;
+        for (; k + 192 < n4; k += 256) {  // four independent loads in flight
+            const v4f a = s[k], b = s[k + 64], c = s[k + 128], e = s[k + 192];
+            if (COPY) o[k] = a, o[k + 64] = b, o[k + 128] = c, o[k + 192] = e;
+            take(a, 0), take(b, 1), take(c, 2), take(e, 3);
+        }
+        for (; k < n4; k += 64) {
+            const v4f a = s[k];
+            if (COPY) o[k] = a;
+            take(a, 0);
+        }
+        s1 = (p1[0] + p1[1]) + (p1[2] + p1[3]);
+        s2 = (p2[0] + p2[1]) + (p2[2] + p2[3]);
+    } else {
+        for (int k = lane; k < d; k += 64) {
+            const float v = src[k];
+            if (COPY) dst[k] = v;
+            s1 += v;
+            s2 += v * v;
+        }
+    }
+    const float inv_d = 1.0f / (float)d;
+    float mu = 0.f, rstd = 1.f;
+    if (norm_kind == NORM_RMS) {
+        rstd = 1.0f / sqrtf(wave_sum_f(s2) * inv_d + kNormEps);
+    } else if (norm_kind == NORM_CENTERED) {
+        mu = wave_sum_f(s1) * inv_d;
+        float q = 0.f;
+        if (VEC) {
+            const int n4 = d >> 2;
+            const v4f* s = reinterpret_cast<const v4f*>(src);
+            float q4[4] = {0.f, 0.f, 0.f, 0.f};
+            auto take = [&](const v4f& v, int i) {
+                const v4f c = v - mu;
+                q4[i] += (c.x * c.x + c.y * c.y) + (c.z * c.z + c.w * c.w);
+            };
+            int k = lane;
+            for (; k + 192 < n4; k += 256) {
+                const v4f a = s[k], b = s[k + 64], c = s[k + 128], e = s[k + 192];
+                take(a, 0), take(b, 1), take(c, 2), take(e, 3);
+            }
+            for (; k < n4; k += 64) take(s[k], 0);
+            q = (q4[0] + q4[1]) + (q4[2] + q4[3]);
+        } else {
+            for (int k = lane; k < d; k += 64) {
+                const float c = src[k] - mu;
+                q += c * c;
+            }
+        }
+        rstd = 1.0f / sqrtf(wave_sum_f(q) * inv_d + kNormEps);
+    }
+    if (lane == 0) {
+        stats[2 * (size_t)r] = mu;
+        stats[2 * (size_t)r + 1] = rstd;
+        if (COPY && coeff != nullptr && routed_coeff != nullptr) routed_coeff[r] = coeff[t];
+    }
+}
+
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void gather_kernel(int T, int d, const float* __restrict__ buf,
                                                           const int* __restrict__ pos, float* __restrict__ out,
@@ -412,9 +505,29 @@ hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream) {
     return hipGetLastError();
 }
 
+hipError_t launch_row_stats(float* stats, const float* in, int rows, int d, int norm_kind, hipStream_t stream) {
+    if (rows <= 0) return hipSuccess;
+    if (vec_ok(d, {in}))
+        scatter_stats_kernel<true, false><<<row_grid(rows), kThreads, 0, stream>>>(rows, d, in, nullptr, nullptr, nullptr,
+                                                                                   nullptr, stats, norm_kind);
+    else
+        scatter_stats_kernel<false, false><<<row_grid(rows), kThreads, 0, stream>>>(rows, d, in, nullptr, nullptr, nullptr,
+                                                                                    nullptr, stats, norm_kind);
+    return hipGetLastError();
+}
+
 hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, const int* pos, float* routed,
-                          float* routed_coeff, hipStream_t stream) {
+                          float* routed_coeff, hipStream_t stream, float* row_stats, int norm_kind) {
     if (T <= 0) return hipSuccess;
+    if (row_stats != nullptr) {
+        if (vec_ok(d, {x, routed}))
+            scatter_stats_kernel<true, true><<<row_grid(T), kThreads, 0, stream>>>(T, d, x, coeff, pos, routed, routed_coeff,
+                                                                                   row_stats, norm_kind);
+        else
+            scatter_stats_kernel<false, true><<<row_grid(T), kThreads, 0, stream>>>(T, d, x, coeff, pos, routed, routed_coeff,
+                                                                                    row_stats, norm_kind);
+        return hipGetLastError();
+    }
     if (vec_ok(d, {x, routed}))
         scatter_kernel<true><<<row_grid(T), kThreads, 0, stream>>>(T, d, x, coeff, pos, routed, routed_coeff);
     else

@@ -26,14 +26,19 @@ __global__ void expert_gemm_generic_kernel(GemmProblem p, int rows, size_t weigh
     const float* b0 = p.B + w0 + (size_t)col * p.K;
     float s0 = 0.f, s1 = 0.f;
     for (int k = 0; k < p.K; ++k) s0 += a[k] * b0[k];
-    if (p.epilogue == EPI_GATED_GELU) {
-        const float* b1 = p.B1 + w0 + (size_t)col * p.K;
-        for (int k = 0; k < p.K; ++k) s1 += a[k] * b1[k];
-        s0 = gelu_dot(s0, s1);
-    } else if (p.epilogue == EPI_RELU) {
-        s0 = fmaxf(s0, 0.f);
-    } else {
+    if (p.epilogue == EPI_RESIDUAL) {
         s0 += p.R[idx];
+    } else {
+        const float mu = p.row_stats ? p.row_stats[2 * (size_t)row] : 0.f, rstd = p.row_stats ? p.row_stats[2 * (size_t)row + 1] : 1.f;
+        s0 = rstd * (s0 - mu * (p.colsum ? p.colsum[w0 + col] : 0.f));
+        if (p.epilogue == EPI_GATED_GELU) {
+            const float* b1 = p.B1 + w0 + (size_t)col * p.K;
+            for (int k = 0; k < p.K; ++k) s1 += a[k] * b1[k];
+            s1 = rstd * (s1 - mu * (p.colsum1 ? p.colsum1[w0 + col] : 0.f));
+            s0 = gelu_dot(s0, s1);
+        } else {
+            s0 = fmaxf(s0, 0.f);
+        }
     }
     p.C[idx] = s0;
 }
@@ -54,7 +59,13 @@ size_t lds_bytes(bool gated, int a_alloc_rows, int K) {
 bool fast_path_ok(const GemmProblem& p) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B) |
                            reinterpret_cast<uintptr_t>(p.B1);
-    return p.K % 32 == 0 && (bits & 15) == 0;
+    return p.K % 32 == 0 && (bits & 15) == 0 && (reinterpret_cast<uintptr_t>(p.row_stats) & 7) == 0;
+}
+
+// the second product needs its residual, the two-matrix form its second matrix
+bool operands_ok(const GemmProblem& p) {
+    if (p.epilogue == EPI_RESIDUAL) return p.R != nullptr;
+    return p.epilogue != EPI_GATED_GELU || p.B1 != nullptr;
 }
 
 }  // namespace
@@ -66,6 +77,7 @@ bool expert_gemm_grouped_ok(const GemmProblem& p, size_t weight_stride) {
 hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t weight_stride, const int* row_expert,
                                                 int rows, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
+    if (!operands_ok(p)) return hipErrorInvalidValue;
     const size_t n = (size_t)rows * p.N;
     expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows, weight_stride, row_expert);
     return hipGetLastError();
@@ -74,6 +86,7 @@ hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t wei
 hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
     if (tile_rows <= 0 || tile_rows % 16 != 0 || tile_rows > gemm_tile_rows(p.epilogue)) return hipErrorInvalidValue;
+    if (!operands_ok(p)) return hipErrorInvalidValue;
     if (!fast_path_ok(p)) {
         const size_t n = (size_t)rows * p.N;
         expert_gemm_generic_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(p, rows, 0, nullptr);
@@ -85,19 +98,22 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hip
     const bool gated = p.epilogue == EPI_GATED_GELU;
     const size_t lds = lds_bytes(gated, a_alloc, p.K);
     return gated ? expert_gemm_launch_one_gated(p, rows, tile, a_alloc, grid, lds, stream)
-                 : expert_gemm_launch_one(p, rows, tile, a_alloc, grid, lds, stream);
+           : p.epilogue == EPI_RELU ? expert_gemm_launch_one_relu(p, rows, tile, a_alloc, grid, lds, stream)
+                                    : expert_gemm_launch_one(p, rows, tile, a_alloc, grid, lds, stream);
 }
 
 hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
                                       const int* sched, int max_tiles, hipStream_t stream) {
     if (max_tiles <= 0) return hipSuccess;
-    if (!expert_gemm_grouped_ok(p, weight_stride)) return hipErrorInvalidValue;  // see launch_expert_gemm_any_shape_grouped
+    if (!expert_gemm_grouped_ok(p, weight_stride) || !operands_ok(p)) return hipErrorInvalidValue;  // see launch_expert_gemm_any_shape_grouped
     const int n_col_tiles = (p.N + kGemmColumns - 1) / kGemmColumns;
     const dim3 grid((unsigned)kXcdCount * (unsigned)xcd_tile_capacity(max_tiles) * (unsigned)n_col_tiles);
     const bool gated = p.epilogue == EPI_GATED_GELU;
     const size_t lds = lds_bytes(gated, gated ? kGemmTileRowsGated : kGemmTileRows, p.K);
     return gated ? expert_gemm_launch_grouped_gated(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream)
-                 : expert_gemm_launch_grouped(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream);
+           : p.epilogue == EPI_RELU
+               ? expert_gemm_launch_grouped_relu(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream)
+               : expert_gemm_launch_grouped(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream);
 }
 
 }  // namespace infmoe

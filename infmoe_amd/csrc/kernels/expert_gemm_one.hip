@@ -1,14 +1,14 @@
-// One of the four instantiations of the matrix-core expert kernel (see expert_gemm_parts.h).
+// One of the six instantiations of the matrix-core expert kernel (see expert_gemm_parts.h).
 #include "expert_gemm_parts.h"
 #include "expert_gemm_tile.h"
 
 namespace infmoe {
 
-hipError_t expert_gemm_launch_one(const GemmProblem& p, int rows, int tile_rows, int a_alloc_rows, dim3 grid,
-                                  size_t lds, hipStream_t stream) {
-    const hipError_t err = allow_lds_once<expert_gemm_kernel<kGemmColumns, false>>(kLdsPerCu);
+hipError_t expert_gemm_launch_one(const GemmProblem& p, int rows, int tile_rows, int a_alloc_rows, dim3 grid, size_t lds,
+                                  hipStream_t stream) {
+    const hipError_t err = allow_lds_once<expert_gemm_kernel<kGemmColumns, EPI_RESIDUAL>>(kLdsPerCu);
     if (err != hipSuccess) return err;
-    expert_gemm_kernel<kGemmColumns, false><<<grid, kGemmThreads, lds, stream>>>(p, rows, tile_rows, a_alloc_rows);
+    expert_gemm_kernel<kGemmColumns, EPI_RESIDUAL><<<grid, kGemmThreads, lds, stream>>>(p, rows, tile_rows, a_alloc_rows);
     return hipGetLastError();
 }
 

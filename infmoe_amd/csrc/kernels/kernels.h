@@ -113,8 +113,10 @@ hipError_t launch_expert_count_static(int T, int E, const int* sel, int* pos, in
 hipError_t launch_fill_i32(int* dst, int n, int value, hipStream_t stream);
 
 // ---- scatter / gather / mix (replaces plugin/cuda/moe.cu:214-258)
+// row_stats: null, or [T][2] that receives launch_row_stats' numbers (norm_kind) for every routed row
 hipError_t launch_scatter(int T, int d, const float* x, const float* coeff, const int* pos, float* routed,
-                          float* routed_coeff, hipStream_t stream);
+                          float* routed_coeff, hipStream_t stream, float* row_stats = nullptr,
+                          int norm_kind = NORM_NONE);
 // routed_coeff: null, or [T]; a routed row whose coefficient is NaN (a token the gating could not score) is
 // written as NaN in full
 hipError_t launch_gather(int T, int d, const float* buf, const int* pos, float* out, hipStream_t stream,
@@ -129,11 +131,25 @@ hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const f
                            size_t gamma_stride, const int* row_expert, int norm_kind, hipStream_t stream,
                            const int* expert_slot = nullptr);
 
+// Row statistics of the norm: stats[r] = (mu_r, rstd_r) with mu_r = 0 and rstd_r = rsqrt(mean(x^2) + eps) for
+// the rms form, the mean and rsqrt(biased variance + eps) for the centered one (two exact passes).  The
+// scatter of the layer computes the same numbers, by the same device code, while it copies the rows.
+hipError_t launch_row_stats(float* stats, const float* in, int rows, int d, int norm_kind, hipStream_t stream);
+
+// In place: w[n][k] *= gamma[k] for the n_rows rows of a [n_rows][d] weight matrix, and colsum[n] = the sum of
+// the scaled row (what the norm-carrying first product wants of an expert's input-side weights).
+hipError_t launch_fold_gamma(float* w, float* colsum, const float* gamma, int n_rows, int d, hipStream_t stream);
+
 // ---- expert GEMMs (replace the three cublasSgemm_v2 calls, fused_gelu_dot_gpu and the D2D
 //      residual copy of plugin/sublayers/T5FFLayer.cc:112-138)
+// The first product of the feed-forward block can carry the block's row norm with it (plugin/sublayers/
+// T5FFLayer.cc:99-103 runs the norm as a launch of its own and keeps the normed rows in memory): with weights
+// whose columns were multiplied by gamma (launch_fold_gamma), the row statistics (mu_r, rstd_r) of
+// launch_row_stats and colsum_n = sum_k gamma_k w_nk, the product of the normed rows with the plain weights
+// is P = rstd_r * (A*B^T - mu_r * colsum_n) on the raw rows A.  Without row statistics P = A*B^T.
 enum Epilogue : int32_t {
-    EPI_RELU = 0,        // C = max(A*B^T, 0)
-    EPI_GATED_GELU = 1,  // C = gelu_tanh(A*B0^T) * (A*B1^T)
+    EPI_RELU = 0,        // C = max(P, 0)
+    EPI_GATED_GELU = 1,  // C = gelu_tanh(P0) * P1
     EPI_RESIDUAL = 2     // C = R + A*B^T
 };
 struct GemmProblem {
@@ -144,6 +160,12 @@ struct GemmProblem {
     float* C;          // [rows][N]
     int N, K;
     int epilogue;
+    // EPI_RELU / EPI_GATED_GELU with the norm carried along: row_stats [rows][2] = (mu, rstd) per row of A, and
+    // for the centered form colsum [N] (colsum1 for B1) - in grouped launches those of expert 0, the others
+    // follow at weight_stride like B.  All null: the plain product.
+    const float* row_stats;
+    const float* colsum;
+    const float* colsum1;
     // grouped launches only: null, or [E] where expert e's weights are at B + expert_slot[e] * weight_stride
     // instead of B + e * weight_stride (experts held in slots in whatever order they arrived)
     const int* expert_slot;

@@ -130,6 +130,7 @@ struct MoELayer::Carve {
     void* countScratch = nullptr;
     float* gateScratch = nullptr;  // partial scores of the gating kernel's slices
     float *coeff = nullptr, *routedCoeff = nullptr, *routed = nullptr, *post = nullptr;
+    float* rowStats = nullptr;  // (mean, reciprocal deviation) of every routed row, when the sub-layer asks for them
     size_t total = 0;
 };
 
@@ -139,7 +140,7 @@ struct MoELayer::Carve {
 // calls cannot.
 //   sub-layer scratch for T rows, shared by all experts because their rows are disjoint
 //     (the reference sizes one full-T scratch per slot, :256-263)
-//   sel[T] pos[T] rowExpert[T] | row tiles | scan scratch | coeff[T] routedCoeff[T] | routed[T][d] | post[T][d]
+//   sel[T] pos[T] rowExpert[T] | row tiles | scan scratch | coeff[T] routedCoeff[T] rowStats[T][2] | routed[T][d] | post[T][d]
 //   (the reference also keeps the T x E score matrix, :246; the fused gating never stores it)
 Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     char* base = static_cast<char*>(workspace);
@@ -162,6 +163,7 @@ Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     c->gateScratch = reinterpret_cast<float*>(take(sizeof(float) * gate_scratch_floats(T, d, E)));
     c->coeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
     c->routedCoeff = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T));
+    c->rowStats = mSublayer->rowStatsKind() != NORM_NONE ? reinterpret_cast<float*>(take(sizeof(float) * 2 * (size_t)T)) : nullptr;
     c->routed = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T * d));
     c->post = reinterpret_cast<float*>(take(sizeof(float) * (size_t)T * d));
     c->total = off;
@@ -358,14 +360,15 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, c.tiles, c.sched,
                                    mSublayer->rowTileHeight(), skinnyMax, c.rowExpert, stream));
     INFMOE_TRY(mark(2));
-    INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream));  // experts see the raw input (:354)
+    // experts see the raw input (:354); the statistics of their row norm are taken while the rows are copied
+    INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream, c.rowStats, mSublayer->rowStatsKind()));
     INFMOE_HIP(hipEventRecord(mRoutingDone, stream));
     INFMOE_TRY(mark(3));
 
     // 4. experts                                                   plugin/MoELayerPlugin.cc:360-402
     GroupedRun g;
     g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
-    g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert;
+    g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert, g.rowStats = c.rowStats;
     g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
     if (skinnyMax > 0) {
         // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
@@ -550,7 +553,8 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedR
             // shared scratch (row stride applied: the public reference omits it at :373,391-392)
             INFMOE_TRY(mSublayer->runInLayer(T, count[e], slotPtr, c.routed + (size_t)offset[e] * d,
                                              c.post + (size_t)offset[e] * d,
-                                             c.subWs + mSublayer->workspaceOffset(offset[e]), cs));
+                                             c.subWs + mSublayer->workspaceOffset(offset[e]), cs,
+                                             c.rowStats ? c.rowStats + 2 * (size_t)offset[e] : nullptr));
             INFMOE_HIP(hipEventRecord(mComputeDone[k], cs));
             lastUse[slot] = k;
             ++k;

@@ -51,7 +51,8 @@ Status MoESubLayer::runGrouped(const GroupedRun& g) {
         const size_t owner = slots ? (size_t)g.expertSlotHost[e] : (size_t)e;
         INFMOE_TRY(runInLayer(g.tokenCount, count[e], weights ? weights + stride * owner : nullptr,
                               g.input + (size_t)offset[e] * d, g.output + (size_t)offset[e] * d,
-                              static_cast<char*>(g.workspace) + workspaceOffset(offset[e]), g.stream));
+                              static_cast<char*>(g.workspace) + workspaceOffset(offset[e]), g.stream,
+                              g.rowStats ? g.rowStats + 2 * (size_t)offset[e] : nullptr));
     }
     return INFMOE_OK;
 }

@@ -29,14 +29,19 @@ size_t T5FFLayer::weightBytes(int d, int h, int ffnKind) {
 }
 
 size_t T5FFLayer::workspaceBytes(int rows, int d, int h) {
-    return sizeof(float) * (size_t)rows * ((size_t)d + (size_t)h);
+    return sizeof(float) * (size_t)rows * ((size_t)d + (size_t)h);  // normed rows, hidden rows
 }
 
-size_t T5FFLayer::weightSize() { return weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind); }
-
-size_t T5FFLayer::workspaceSize(int32_t tokenCount) {
-    return align_up(workspaceBytes(tokenCount, mEmbeddingSize, mHiddenSize));
+// A device slot holds the expert's arrays in the reference's order and, behind them, the column sums of the
+// input-side matrices after gamma has been multiplied into them (one or two arrays of h floats).
+size_t T5FFLayer::weightSize() {
+    return weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind) + sizeof(float) * (size_t)(nMatrices() - 1) * mHiddenSize;
 }
+
+// In a layer: hidden rows, then room for (mu, rstd, -, -) per row, used when nobody hands the statistics over.
+size_t T5FFLayer::layerWorkspaceBytes(int rows) const { return sizeof(float) * (size_t)rows * ((size_t)mHiddenSize + 4); }
+
+size_t T5FFLayer::workspaceSize(int32_t tokenCount) { return align_up(layerWorkspaceBytes(tokenCount)); }
 
 int T5FFLayer::keyIndex(const char* key, size_t* off, size_t* cnt) const {
     const size_t d = mEmbeddingSize, dh = (size_t)mEmbeddingSize * mHiddenSize;
@@ -59,7 +64,7 @@ Status T5FFLayer::ensureHostStore() {
     if (mHostWeights != nullptr) return INFMOE_OK;
     // page-locked like the reference's npz store (plugin/thirdparty/cnpy/cnpy.h:27-39), so that
     // hipMemcpyAsync from it really is asynchronous
-    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mHostWeights), slotStride() * (size_t)mExpertCount,
+    INFMOE_HIP(hipHostMalloc(reinterpret_cast<void**>(&mHostWeights), hostStride() * (size_t)mExpertCount,
                              hipHostMallocDefault));
     mHave.assign((size_t)mExpertCount * (nMatrices() + 1), 0);
     return INFMOE_OK;
@@ -74,13 +79,16 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     // the reference asserts on the byte count of every array (plugin/sublayers/T5FFLayer.cc:62,69,76,83)
     if (count != cnt) return fail(INFMOE_ERR_INVALID_ARGUMENT, "%s: expected %zu floats, got %zu", key, cnt, count);
     INFMOE_TRY(ensureHostStore());
-    float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)expert);
+    float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + hostStride() * (size_t)expert);
     memcpy(slot + off, host, cnt * sizeof(float));
     mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
     mVersion.fetch_add(1, std::memory_order_acq_rel);
-    if (mDeviceWeights != nullptr) {  // already resident: keep the device copy in step (blocking; not a hot path)
-        char* dev = static_cast<char*>(mDeviceWeights) + slotStride() * (size_t)expert + off * sizeof(float);
-        INFMOE_HIP(hipMemcpy(dev, slot + off, cnt * sizeof(float), hipMemcpyHostToDevice));
+    if (mDeviceWeights != nullptr) {
+        // already resident: the device slot is made anew from the host store, because gamma is multiplied into
+        // the input-side matrices there and either may be the array that changed (blocking; not a hot path)
+        INFMOE_HIP(hipDeviceSynchronize());
+        INFMOE_TRY(copyWeights(static_cast<char*>(mDeviceWeights) + deviceStride() * (size_t)expert, expert, nullptr));
+        INFMOE_HIP(hipStreamSynchronize(nullptr));
     }
     return INFMOE_OK;
 }
@@ -94,7 +102,7 @@ Status T5FFLayer::loadFromFile() {
     const char* const* keys = mFfnKind == FFN_GATED_GELU ? kGated : kRelu;
     const size_t d = mEmbeddingSize, h = mHiddenSize;
     for (int e = 0; e < mExpertCount; ++e) {
-        float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + slotStride() * (size_t)e);
+        float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + hostStride() * (size_t)e);
         for (int j = 0; j <= nMatrices(); ++j) {
             size_t off = 0, cnt = 0;
             keyIndex(keys[j], &off, &cnt);
@@ -148,18 +156,34 @@ void T5FFLayer::terminate() {
 Status T5FFLayer::makeResident() {
     if (mDeviceWeights != nullptr) return INFMOE_OK;
     if (mHostWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: makeResident before initialize");
-    const size_t bytes = slotStride() * (size_t)mExpertCount;
-    INFMOE_HIP(hipMalloc(&mDeviceWeights, bytes));
-    INFMOE_HIP(hipMemcpy(mDeviceWeights, mHostWeights, bytes, hipMemcpyHostToDevice));
+    INFMOE_HIP(hipMalloc(&mDeviceWeights, deviceStride() * (size_t)mExpertCount));
+    for (int e = 0; e < mExpertCount; ++e) {
+        const Status s = copyWeights(static_cast<char*>(mDeviceWeights) + deviceStride() * (size_t)e, e, nullptr);
+        if (s != INFMOE_OK) {
+            (void)hipFree(mDeviceWeights);
+            mDeviceWeights = nullptr;
+            return s;
+        }
+    }
+    INFMOE_HIP(hipStreamSynchronize(nullptr));
     return INFMOE_OK;
 }
 
 Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
-    // plugin/sublayers/T5FFLayer.cc:55-88 issues four copies; the host store is already packed in
-    // slot order, so one copy moves the expert.
+    // plugin/sublayers/T5FFLayer.cc:55-88 issues four copies; the host store is already packed in slot order,
+    // so one copy moves the expert.  Then, on the same stream, the norm's gamma is multiplied into the
+    // input-side matrices where they now lie and their column sums are put behind the arrays: the first
+    // product of the expert then carries the norm with it (a read and a write of those matrices in device
+    // memory, a few percent of what the copy over the host link takes).
     if (mHostWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: copyWeights before initialize");
-    const char* src = reinterpret_cast<const char*>(mHostWeights) + slotStride() * (size_t)expert;
-    INFMOE_HIP(hipMemcpyAsync(dst, src, weightSize(), hipMemcpyHostToDevice, stream));
+    const char* src = reinterpret_cast<const char*>(mHostWeights) + hostStride() * (size_t)expert;
+    const int d = mEmbeddingSize, h = mHiddenSize;
+    INFMOE_HIP(hipMemcpyAsync(dst, src, weightBytes(d, h, mFfnKind), hipMemcpyHostToDevice, stream));
+    float* w = static_cast<float*>(dst);
+    const size_t dh = (size_t)d * h;
+    float* colsum = w + d + (size_t)nMatrices() * dh;
+    for (int m = 0; m < nMatrices() - 1; ++m)
+        INFMOE_HIP(launch_fold_gamma(w + d + m * dh, colsum + (size_t)m * h, w, h, d, stream));
     return INFMOE_OK;
 }
 
@@ -172,23 +196,44 @@ int T5FFLayer::skinnyMaxRows(int32_t tokenCount) const {
     return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kSkinnyMaxRows : 0;
 }
 
+// folded: `weights` is a slot as copyWeights leaves it (gamma multiplied into the input-side matrices, column
+// sums behind the arrays), the workspace is the in-layer one, and the norm rides on the first product; rowStats
+// are the rows' (mu, rstd) or null to compute them here.  Not folded: `weights` holds the arrays as the caller
+// made them (plugin/sublayers/T5FFLayer.cc:100-131), the norm is a launch of its own into the workspace.
 Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int h, int normKind, int ffnKind,
-                         const void* weights, const float* in, float* out, void* workspace, hipStream_t stream) {
+                         const void* weights, const float* in, float* out, void* workspace, hipStream_t stream,
+                         bool folded, const float* rowStats) {
     if (rows <= 0) return INFMOE_OK;
     const float* w = static_cast<const float*>(weights);
     const size_t dh = (size_t)d * h;
-    float* ln = static_cast<float*>(workspace);
-    float* hid = ln + (size_t)rows * d;
-    // plugin/sublayers/T5FFLayer.cc:99-103
-    INFMOE_HIP(launch_row_norm(ln, in, rows, d, w, 0, nullptr, normKind, stream));
-    GemmProblem g1{};  // plugin/sublayers/T5FFLayer.cc:112-126
-    g1.A = ln, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
+    const int nMat = ffnKind == FFN_GATED_GELU ? 3 : 2;
+    GemmProblem g1{};  // plugin/sublayers/T5FFLayer.cc:99-126: norm, one or two products, activation
+    float* hid = nullptr;
+    if (folded) {
+        hid = static_cast<float*>(workspace);
+        if (rowStats == nullptr) {  // outside a layer call: nobody has looked at the rows yet
+            float* stats = hid + (size_t)rows * h;
+            INFMOE_HIP(launch_row_stats(stats, in, rows, d, normKind, stream));
+            rowStats = stats;
+        }
+        g1.A = in, g1.row_stats = rowStats;
+        if (normKind == NORM_CENTERED) {  // the rms form has no mean to take out
+            g1.colsum = w + d + (size_t)nMat * dh;
+            g1.colsum1 = ffnKind == FFN_GATED_GELU ? g1.colsum + h : nullptr;
+        }
+    } else {
+        float* ln = static_cast<float*>(workspace);
+        hid = ln + (size_t)rows * d;
+        INFMOE_HIP(launch_row_norm(ln, in, rows, d, w, 0, nullptr, normKind, stream));
+        g1.A = ln;
+    }
+    g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
     g1.B1 = ffnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
     g1.epilogue = ffnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
     GemmProblem g2{};  // plugin/sublayers/T5FFLayer.cc:130-138 (residual instead of copy + beta = 1)
-    g2.A = hid, g2.B = w + d + (ffnKind == FFN_GATED_GELU ? 2 : 1) * dh, g2.R = in, g2.C = out, g2.N = d, g2.K = h;
+    g2.A = hid, g2.B = w + d + (size_t)(nMat - 1) * dh, g2.R = in, g2.C = out, g2.N = d, g2.K = h;
     g2.epilogue = EPI_RESIDUAL;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(ln)) & 15) == 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(g1.A) | reinterpret_cast<uintptr_t>(hid)) & 15) == 0;
     const bool skinny = rows <= kSkinnyMaxRows && decode_like(layerTokens, expertCount) && d % 4 == 0 && h % 4 == 0 && aligned;
     if (skinny) {
         INFMOE_HIP(launch_expert_skinny(g1, rows, stream));
@@ -204,30 +249,39 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
 
 Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                       hipStream_t stream) {
-    // outside a layer call the expert stands alone: a call of tokenCount tokens over one expert
+    // outside a layer call the expert stands alone: a call of tokenCount tokens over one expert, on a slot
+    // that copyWeights filled
     return runOne(tokenCount, tokenCount, 1, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
-                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream);
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, true, nullptr);
 }
 
 Status T5FFLayer::runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input,
-                             void* output, void* workspace, hipStream_t stream) {
+                             void* output, void* workspace, hipStream_t stream, const float* rowStats) {
     return runOne(tokenCount, layerTokens, mExpertCount, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
-                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream);
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, true, rowStats);
 }
 
 Status T5FFLayer::runGrouped(const GroupedRun& g) {
     if (mDeviceWeights == nullptr && g.weights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: runGrouped needs resident weights");
     const int T = g.tokenCount, d = mEmbeddingSize, h = mHiddenSize;
-    const size_t dh = (size_t)d * h, stride = (g.weights ? g.weightStride : slotStride()) / sizeof(float);
+    const size_t dh = (size_t)d * h, stride = (g.weights ? g.weightStride : deviceStride()) / sizeof(float);
     const float* w = static_cast<const float*>(g.weights ? g.weights : mDeviceWeights);
     const int* slot = g.weights ? g.expertSlot : nullptr;
-    float* ln = static_cast<float*>(g.workspace);
-    float* hid = ln + (size_t)T * d;
-    INFMOE_HIP(launch_row_norm(ln, g.input, T, d, w, stride, g.rowExpert, mNormKind, g.stream, slot));
+    float* hid = static_cast<float*>(g.workspace);
+    const float* stats = g.rowStats;
+    if (stats == nullptr) {  // a caller that did not compute them with the scatter
+        float* own = hid + (size_t)T * h;
+        INFMOE_HIP(launch_row_stats(own, g.input, T, d, mNormKind, g.stream));
+        stats = own;
+    }
     GemmProblem g1{};
     g1.expert_slot = slot;
-    g1.A = ln, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
+    g1.A = g.input, g1.row_stats = stats, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
     g1.B1 = mFfnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
+    if (mNormKind == NORM_CENTERED) {  // the rms form has no mean to take out
+        g1.colsum = w + d + (size_t)nMatrices() * dh;
+        g1.colsum1 = mFfnKind == FFN_GATED_GELU ? g1.colsum + h : nullptr;
+    }
     g1.epilogue = mFfnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
     GemmProblem g2{};
     g2.expert_slot = slot;

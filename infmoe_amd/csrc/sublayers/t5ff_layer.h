@@ -8,8 +8,12 @@
 //         "relu" with wi, wo (the dense_relu_dense the layer is named after).
 // Device slot of one expert, as plugin/sublayers/T5FFLayer.cc:100,112,118-119,130-131:
 //   [gamma d | wi h*d | wo d*h]  or  [gamma d | wi_0 h*d | wi_1 h*d | wo d*h]   (floats)
-// Workspace for M rows: [LN M*d | H M*h] (the reference keeps two M*h buffers; the gelu*mul
-// product is formed in the GEMM epilogue here, so one is enough).
+// As copyWeights leaves it, gamma is multiplied into the input-side matrices and their column sums follow the
+// arrays: the norm then rides on the first product (rstd_r * (x.w' - mu_r * colsum)) and is no launch of its own.
+// Workspace for M rows in a layer: [H M*h | row statistics M*4] (the reference keeps the normed rows M*d and two
+// M*h buffers; here the gelu*mul product is formed in the epilogue, so one hidden buffer is all; the statistics
+// area is used when nobody hands them over).  infmoe_t5ff_run, which takes the arrays as the caller made them,
+// runs the norm as a launch of its own into [LN M*d | H M*h].
 #pragma once
 
 #include <atomic>
@@ -29,12 +33,13 @@ class T5FFLayer : public MoESubLayer {
                              int32_t nbOutputs) override;
     size_t weightSize() override;
     size_t workspaceSize(int32_t tokenCount) override;
-    size_t workspaceOffset(int32_t firstRow) override { return workspaceBytes(firstRow, mEmbeddingSize, mHiddenSize); }
+    size_t workspaceOffset(int32_t firstRow) override { return layerWorkspaceBytes(firstRow); }
     Status copyWeights(void* dst, int expert, hipStream_t stream) override;
     Status run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                hipStream_t stream) override;
     Status runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input, void* output,
-                      void* workspace, hipStream_t stream) override;
+                      void* workspace, hipStream_t stream, const float* rowStats) override;
+    int rowStatsKind() const override { return mNormKind; }
     Status initialize() override;
     void terminate() override;
 
@@ -42,7 +47,7 @@ class T5FFLayer : public MoESubLayer {
     uint64_t weightsVersion() const override { return mVersion.load(std::memory_order_acquire); }
     Status makeResident() override;
     const void* residentWeights() const override { return mDeviceWeights; }
-    size_t residentStride() const override { return slotStride(); }
+    size_t residentStride() const override { return deviceStride(); }
     int skinnyMaxRows(int32_t tokenCount) const override;
     int rowTileHeight() const override { return mFfnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
     Status runGrouped(const GroupedRun& g) override;
@@ -51,17 +56,22 @@ class T5FFLayer : public MoESubLayer {
     static size_t weightBytes(int d, int h, int ffnKind);
     static size_t workspaceBytes(int rows, int d, int h);
     static Status runOne(int rows, int layerTokens, int expertCount, int d, int h, int normKind, int ffnKind,
-                         const void* weights, const float* in, float* out, void* workspace, hipStream_t stream);
+                         const void* weights, const float* in, float* out, void* workspace, hipStream_t stream,
+                         bool folded, const float* rowStats);
 
    private:
     int mNormKind, mFfnKind;
     int nMatrices() const { return mFfnKind == FFN_GATED_GELU ? 3 : 2; }
-    size_t slotStride() const { return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind)); }
+    size_t hostStride() const { return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind)); }
+    size_t deviceStride() const {
+        return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind) + sizeof(float) * (size_t)(nMatrices() - 1) * mHiddenSize);
+    }
+    size_t layerWorkspaceBytes(int rows) const;
     int keyIndex(const char* key, size_t* offsetFloats, size_t* countFloats) const;
     Status ensureHostStore();
     Status loadFromFile();
 
-    float* mHostWeights = nullptr;   // page-locked, E slots of slotStride() bytes
+    float* mHostWeights = nullptr;   // page-locked, E slots of hostStride() bytes
     std::vector<uint8_t> mHave;      // [E][nMatrices+1] which arrays have been provided
     void* mDeviceWeights = nullptr;  // E slots when resident
     std::atomic<uint64_t> mVersion{0};  // bumped by every setWeights
