@@ -213,14 +213,14 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
 
+    # (the expert norm is no phase of its own: it rides on the first expert product)
     # the bandwidth-bound phases: algorithmic bytes / phase time (the phase times include the launch
     # gaps and the event marks, a few microseconds each), against the HBM peak
     cpm2 = cfg["variant"] == "cpm_2"
     mix = cfg["variant"] == "base_layer"
     phase_bytes = {
         "gating": 4.0 * (T * d + E * d + (d if cpm2 else 0) + 2 * T),
-        "scatter": 4.0 * (2 * T * d + T + (2 * T if mix else 0)),
-        "expert_norm": 4.0 * (2 * T * d + d),
+        "scatter": 4.0 * (2 * T * d + T + 2 * T + (2 * T if mix else 0)),  # rows, pos, row statistics, coefficients
         "gather": 4.0 * ((3 * T * d + 2 * T) if mix else (2 * T * d + T)),
     }
     phase_rates = {k: {"bytes": v, "GB/s": round(v / (phases[k] * 1e-3) / 1e9, 1),
