@@ -28,11 +28,12 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 PCIE_PEAK_GBS = 64.0           # host link, PCIe Gen5 x16, one direction
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # benchmark scaled by what the same counters read for the row-copy kernels of known size
-# (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt).  Counters cannot be read from inside a run.
-# Kept as the ratio counter bytes / algorithmic bytes of the profiled launch (c2: 5.74 GB against 5.52 GB of
-# weights and activations; c5: 4.04 GB against 4.03 GB of weights of 24 active experts) and applied to the
-# algorithmic bytes of the run at hand, whose number of active experts may differ.
-MEASURED_TRAFFIC_RATIO = {"c2": 5.74 / 5.52, "c5": 4.04 / 4.03}
+# (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt;
+# counters cannot be read from inside a run).  Kept as the ratio counter bytes / algorithmic bytes of the
+# profiled launches (c2: 5.72 GB on average over the two launches against 5.60 GB of weights and
+# activations; c5: 4.03 GB against 4.03 GB of weights of 24 active experts) and applied to the algorithmic
+# bytes of the run at hand, whose number of active experts may differ.
+MEASURED_TRAFFIC_RATIO = {"c2": 5.72 / 5.60, "c5": 4.03 / 4.03}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
@@ -213,7 +214,8 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
 
-    # (the expert norm is no phase of its own: it rides on the first expert product)
+    # (with the rms norm of every workload here the expert norm is no phase of its own: it rides on the first
+    # expert product)
     # the bandwidth-bound phases: algorithmic bytes / phase time (the phase times include the launch
     # gaps and the event marks, a few microseconds each), against the HBM peak
     cpm2 = cfg["variant"] == "cpm_2"

@@ -161,7 +161,8 @@ int32_t infmoe_last_streaming(infmoe_plugin* p, int32_t* copies, int32_t* hits);
  * python/examples/stacked_moe.py:55-60).  When enabled, infmoe_enqueue records HIP events on its
  * stream at the phase boundaries; infmoe_last_timing waits for the last call and returns the
  * elapsed milliseconds of: [0] gating, [1] count+sort, [2] scatter (with the row statistics of the expert
- * norm), [3] what a sub-layer does before its first product (T5_FF: nothing, its norm is folded into it),
+ * norm), [3] what a sub-layer does before its first product (T5_FF: nothing with the rms norm, which rides on
+ * that product; the row norm with the centered one),
  * [4] first expert GEMM (norm and activation fused), [5] second expert GEMM (residual fused),
  * [6] gather / mix.  Phases 3-5 are only separated when all experts are resident (otherwise the
  * whole streamed expert loop is reported in [4]).  `ms` holds INFMOE_N_PHASES floats.

@@ -29,12 +29,12 @@ __global__ void expert_gemm_generic_kernel(GemmProblem p, int rows, size_t weigh
     if (p.epilogue == EPI_RESIDUAL) {
         s0 += p.R[idx];
     } else {
-        const float mu = p.row_stats ? p.row_stats[2 * (size_t)row] : 0.f, rstd = p.row_stats ? p.row_stats[2 * (size_t)row + 1] : 1.f;
-        s0 = rstd * (s0 - mu * (p.colsum ? p.colsum[w0 + col] : 0.f));
+        const float rstd = p.row_stats ? p.row_stats[2 * (size_t)row + 1] : 1.f;
+        s0 *= rstd;
         if (p.epilogue == EPI_GATED_GELU) {
             const float* b1 = p.B1 + w0 + (size_t)col * p.K;
             for (int k = 0; k < p.K; ++k) s1 += a[k] * b1[k];
-            s1 = rstd * (s1 - mu * (p.colsum1 ? p.colsum1[w0 + col] : 0.f));
+            s1 *= rstd;
             s0 = gelu_dot(s0, s1);
         } else {
             s0 = fmaxf(s0, 0.f);

@@ -74,17 +74,16 @@ __device__ __forceinline__ void static_for(F&& f) {
 // an 8-k group and their sums meet in the epilogue).  The instruction takes the B operand exactly as
 // the 32x32x2 form holds it (lane -> column lane % 32, float4 lane / 32), so a group costs one more
 // LDS read per k group and four short instructions: rows are padded to 4, not to 16.
-// EPI: the epilogue.  EPI_RESIDUAL adds R to the product.  EPI_RELU / EPI_GATED_GELU can carry the row norm
-// of the T5 feed-forward block (plugin/sublayers/T5FFLayer.cc:99-103) with them: when `stats` is given, A
-// holds the raw rows, B holds weights whose columns were multiplied by the norm's gamma beforehand, and the
-// product becomes rstd_r * (acc - mu_r * colsum_n) before the activation, which is the product of the normed
-// rows with the plain weights (stats: [row][2] = mu, rstd; colsum_n = sum_k gamma_k w_nk, needed only where
-// mu is not 0, i.e. for the centered form; null otherwise).  The inner loop does not know of any of it.
+// EPI: the epilogue.  EPI_RESIDUAL adds R to the product.  EPI_RELU / EPI_GATED_GELU can carry the RMS row
+// norm of the T5 feed-forward block (README.md:115, plugin/sublayers/T5FFLayer.cc:98-103) with them: when
+// `stats` is given, A holds the raw rows, B holds weights whose columns were multiplied by the norm's gamma
+// beforehand, and the product becomes rstd_r * acc before the activation, which is the product of the
+// normed rows with the plain weights (stats: [row][2], of which [1] = rstd_r is used).  The inner loop does
+// not know of any of it.
 template <int NMB, int G4, int BN, int EPI, int BK>
 __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const float* __restrict__ R,
                                           float* __restrict__ C, int rows, const float* __restrict__ B0,
                                           const float* __restrict__ B1, int n0, int N, int K,
-                                          const float* __restrict__ colsum0, const float* __restrict__ colsum1,
                                           const float* __restrict__ stats, float* __restrict__ smem,
                                           int a_alloc_rows) {
     static_assert(BN == 128, "each of the 4 waves owns one 32-column block");
@@ -280,30 +279,20 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     constexpr bool residual = EPI == EPI_RESIDUAL;
     if constexpr (NORM) {
         if (stats != nullptr) {
-            // (mu, rstd) of every row this lane holds, fetched together (clamped, always valid addresses), and the
-            // column sums of this lane's columns; then acc = rstd * (acc - mu * colsum)
-            auto st = [&](int row) { return *reinterpret_cast<const float2*>(stats + 2 * min(row, rows - 1)); };
-            const int c32 = min(n0 + wave * 32 + i32, N - 1);
-            float cs32[NB], cs16[NB][2];
-#pragma unroll
-            for (int m = 0; m < NB; ++m) {
-                const float* cs = m == 0 ? colsum0 : colsum1;
-                cs32[m] = cs != nullptr ? cs[c32] : 0.f;
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) cs16[m][nb] = cs != nullptr ? cs[min(n0 + wave * 32 + 16 * nb + i16, N - 1)] : 0.f;
-            }
+            // rstd of every row this lane holds, fetched together (clamped, always valid addresses)
+            auto st = [&](int row) { return stats[2 * min(row, rows - 1) + 1]; };
 #pragma unroll
             for (int mb = 0; mb < N32; ++mb) {
-                float2 f[16];
+                float f[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) f[r] = st(32 * mb + 8 * (r / 4) + 4 * kh + (r % 4));
 #pragma unroll
                 for (int m = 0; m < NB; ++m)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc32[m][mb][r] = f[r].y * (acc32[m][mb][r] - f[r].x * cs32[m]);
+                    for (int r = 0; r < 16; ++r) acc32[m][mb][r] *= f[r];
             }
             if (T16) {
-                float2 f[4];
+                float f[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) f[r] = st(32 * N32 + 4 * kq + r);
 #pragma unroll
@@ -311,15 +300,12 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
 #pragma unroll
                     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) acc16[m][nb][r] = f[r].y * (acc16[m][nb][r] - f[r].x * cs16[m][nb]);
+                        for (int r = 0; r < 4; ++r) acc16[m][nb][r] *= f[r];
             }
 #pragma unroll
             for (int q = 0; q < G4; ++q)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float2 f = st(TAIL0 + 4 * q + r);
-                    acc4[q][r] = f.y * (acc4[q][r] - f.x * cs32[0]);
-                }
+                for (int r = 0; r < 4; ++r) acc4[q][r] *= st(TAIL0 + 4 * q + r);
         }
     }
     if constexpr (residual) {
@@ -411,9 +397,8 @@ __device__ __forceinline__ TileShape tile_shape(int rows, bool wide) {
 
 template <int BN, int EPI>
 __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, float* C, int rows, const float* B0,
-                                              const float* B1, int n0, int N, int K, const float* colsum0,
-                                              const float* colsum1, const float* stats, float* smem,
-                                              int a_alloc_rows) {
+                                              const float* B1, int n0, int N, int K, const float* stats,
+                                              float* smem, int a_alloc_rows) {
     constexpr bool GATED = EPI == EPI_GATED_GELU;
     // the gated form keeps two accumulator sets, so its tiles are half as tall
     constexpr int kMaxMb = (GATED ? kGemmTileRowsGated : kGemmTileRows) / 16;
@@ -426,14 +411,13 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
         if constexpr ((n) <= kMaxMb && ((g) == 0 || (!GATED && (n) >= 2 && (n) < kMaxMb))) {                    \
             if constexpr (!GATED && 16 * (n) + 4 * (g) <= 16 * kMaxMb64) {                                      \
                 if (wide) {                                                                                     \
-                    gemm_tile<n, g, BN, EPI, 64>(A, R, C, rows, B0, B1, n0, N, K, colsum0, colsum1, stats, smem, \
+                    gemm_tile<n, g, BN, EPI, 64>(A, R, C, rows, B0, B1, n0, N, K, stats, smem,                  \
                                                  min(a_alloc_rows, 16 * kMaxMb64));                             \
                     break;                                                                                      \
                 }                                                                                               \
             }                                                                                                   \
             if constexpr ((g) == 0 || 16 * (n) + 4 * (g) > 16 * kMaxMb64)                                       \
-                gemm_tile<n, g, BN, EPI, 32>(A, R, C, rows, B0, B1, n0, N, K, colsum0, colsum1, stats, smem,    \
-                                             a_alloc_rows);                                                     \
+                gemm_tile<n, g, BN, EPI, 32>(A, R, C, rows, B0, B1, n0, N, K, stats, smem, a_alloc_rows);       \
         }                                                                                                       \
         break;
 #define INFMOE_CASE(n) INFMOE_CASE_G(n, 0) INFMOE_CASE_G(n, 1) INFMOE_CASE_G(n, 2)
@@ -456,7 +440,7 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, in
     const int rows = min(tile_rows, rows_total - row0);
     const int n0 = blockIdx.x * BN;
     gemm_dispatch<BN, EPI>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
-                           p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K, p.colsum, p.colsum1,
+                           p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K,
                            p.row_stats ? p.row_stats + 2 * (size_t)row0 : nullptr, smem, a_alloc_rows);
 }
 
@@ -480,8 +464,6 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProbl
     const float* B1 = GATED ? p.B1 + (size_t)owner * weight_stride : nullptr;
     gemm_dispatch<BN, EPI>(p.A + (size_t)rt.row0 * p.K, p.R ? p.R + (size_t)rt.row0 * p.N : nullptr,
                            p.C + (size_t)rt.row0 * p.N, rt.rows, B0, B1, n0, p.N, p.K,
-                           p.colsum ? p.colsum + (size_t)owner * weight_stride : nullptr,
-                           p.colsum1 ? p.colsum1 + (size_t)owner * weight_stride : nullptr,
                            p.row_stats ? p.row_stats + 2 * (size_t)rt.row0 : nullptr, smem,
                            GATED ? kGemmTileRowsGated : kGemmTileRows);
 }

@@ -56,13 +56,12 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // SEG: 16-byte loads per lane per weight row per chunk; RPN: weight rows loaded together
 // EPI: as in the matrix-core kernel - EPI_RESIDUAL adds R to the product; EPI_RELU and EPI_GATED_GELU carry the
-// block's row norm with them when `stats` is given: the weights then have gamma multiplied in, and a sum
-// becomes rstd_row * (sum - mu_row * colsum_n) before the activation (stats: [row][2] = mu, rstd).
+// block's RMS row norm with them when `stats` is given: the weights then have gamma multiplied in, and a sum
+// becomes rstd_row * sum before the activation (stats: [row][2], of which [1] = rstd_row is used).
 template <int M, int SEG, int RPN, int EPI>
 __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const float* __restrict__ R,
                                             float* __restrict__ C, int rows, const float* __restrict__ B0,
                                             const float* __restrict__ B1, int N, int K,
-                                            const float* __restrict__ colsum0, const float* __restrict__ colsum1,
                                             const float* __restrict__ stats, int row_blocks) {
     constexpr bool GATED = EPI == EPI_GATED_GELU;
     constexpr bool NORM = EPI != EPI_RESIDUAL;
@@ -73,12 +72,9 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
     // the wave index is uniform: as a scalar it lets every row base live in SGPRs, so a load needs
     // only the lane's 32-bit offset instead of a 64-bit address per (row, segment)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    float mu[M], rstd[M];
+    float rstd[M];
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-        mu[m] = NORM && stats != nullptr ? stats[2 * min(m, rows - 1)] : 0.f;
-        rstd[m] = NORM && stats != nullptr ? stats[2 * min(m, rows - 1) + 1] : 1.f;
-    }
+    for (int m = 0; m < M; ++m) rstd[m] = NORM && stats != nullptr ? stats[2 * min(m, rows - 1) + 1] : 1.f;
 #pragma unroll 1
     for (int rb = 0; rb < row_blocks; ++rb) {
     const int n_base = ((blockIdx.x * kWaves + wave) * row_blocks + rb) * RW;
@@ -160,18 +156,14 @@ __device__ __forceinline__ void skinny_body(const float* __restrict__ A, const f
     const int my_m = lane / RW, my_n = n_base + lane % RW;
     float res = 0.f;
     if (residual) res = R[(size_t)min(my_m, rows - 1) * N + min(my_n, N - 1)];
-    // column sums of this block's weight rows (the centered norm's mean term), one per lane % RW, read by index below
-    float cs0 = 0.f, cs1 = 0.f;
-    if (NORM && colsum0 != nullptr) cs0 = colsum0[min(my_n, N - 1)];
-    if (GATED && colsum1 != nullptr) cs1 = colsum1[min(my_n, N - 1)];
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             float v = wave_sum(acc[0][r][m]);
-            if (NORM) v = rstd[m] * (v - mu[m] * __shfl(cs0, r));
+            if (NORM) v *= rstd[m];
             if (GATED)
-                v = gelu_dot(v, rstd[m] * (wave_sum(acc[NB - 1][r][m]) - mu[m] * __shfl(cs1, r)));
+                v = gelu_dot(v, rstd[m] * wave_sum(acc[NB - 1][r][m]));
             else if (residual)
                 v += res;
             else
@@ -192,8 +184,6 @@ __global__ __launch_bounds__(kThreads, EPI == EPI_GATED_GELU ? 2 : 3) void exper
     int rows = rows_fixed, row0 = 0;
     const float* B0 = p.B;
     const float* B1 = p.B1;
-    const float* colsum0 = p.colsum;
-    const float* colsum1 = p.colsum1;
     if (count != nullptr) {
         const int e = blockIdx.y;
         rows = count[e];
@@ -201,8 +191,6 @@ __global__ __launch_bounds__(kThreads, EPI == EPI_GATED_GELU ? 2 : 3) void exper
         const int owner = p.expert_slot ? p.expert_slot[e] : e;
         B0 += (size_t)owner * weight_stride;
         if (GATED) B1 += (size_t)owner * weight_stride;
-        if (colsum0 != nullptr) colsum0 += (size_t)owner * weight_stride;
-        if (colsum1 != nullptr) colsum1 += (size_t)owner * weight_stride;
     }
     if (rows <= 0 || rows > kSkinnyMaxRows) return;
     const float* A = p.A + (size_t)row0 * p.K;
@@ -212,14 +200,14 @@ __global__ __launch_bounds__(kThreads, EPI == EPI_GATED_GELU ? 2 : 3) void exper
     // One body per row count: a row more than needed would cost its loads of the activation chunk
     // again for every block of weight rows (with 5 rows in the 8-row body, 60 % more of them).
     switch (rows) {
-        case 1: skinny_body<1, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 2: skinny_body<2, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 3: skinny_body<3, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 4: skinny_body<4, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 5: skinny_body<5, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 6: skinny_body<6, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        case 7: skinny_body<7, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
-        default: skinny_body<8, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, colsum0, colsum1, stats, row_blocks); break;
+        case 1: skinny_body<1, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 2: skinny_body<2, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 3: skinny_body<3, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 4: skinny_body<4, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 5: skinny_body<5, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 6: skinny_body<6, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 7: skinny_body<7, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        default: skinny_body<8, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
     }
 }
 

@@ -136,17 +136,19 @@ hipError_t launch_row_norm(float* out, const float* in, int rows, int d, const f
 // scatter of the layer computes the same numbers, by the same device code, while it copies the rows.
 hipError_t launch_row_stats(float* stats, const float* in, int rows, int d, int norm_kind, hipStream_t stream);
 
-// In place: w[n][k] *= gamma[k] for the n_rows rows of a [n_rows][d] weight matrix, and colsum[n] = the sum of
-// the scaled row (what the norm-carrying first product wants of an expert's input-side weights).
-hipError_t launch_fold_gamma(float* w, float* colsum, const float* gamma, int n_rows, int d, hipStream_t stream);
+// In place: w[n][k] *= gamma[k] for the n_rows rows of a [n_rows][d] weight matrix (what the norm-carrying
+// first product wants of an expert's input-side weights).
+hipError_t launch_fold_gamma(float* w, const float* gamma, int n_rows, int d, hipStream_t stream);
 
 // ---- expert GEMMs (replace the three cublasSgemm_v2 calls, fused_gelu_dot_gpu and the D2D
 //      residual copy of plugin/sublayers/T5FFLayer.cc:112-138)
-// The first product of the feed-forward block can carry the block's row norm with it (plugin/sublayers/
+// The first product of the feed-forward block can carry the block's RMS row norm with it (plugin/sublayers/
 // T5FFLayer.cc:99-103 runs the norm as a launch of its own and keeps the normed rows in memory): with weights
-// whose columns were multiplied by gamma (launch_fold_gamma), the row statistics (mu_r, rstd_r) of
-// launch_row_stats and colsum_n = sum_k gamma_k w_nk, the product of the normed rows with the plain weights
-// is P = rstd_r * (A*B^T - mu_r * colsum_n) on the raw rows A.  Without row statistics P = A*B^T.
+// whose columns were multiplied by gamma (launch_fold_gamma) and the rows' rstd_r from launch_row_stats, the
+// product of the normed rows with the plain weights is P = rstd_r * (A*B^T) on the raw rows A.  Without row
+// statistics P = A*B^T.  (The centered norm is not carried this way: rstd_r * (A*B^T - mu_r * sum_k B_nk)
+// subtracts two large numbers when a row's mean is large against its deviation, and then loses to the
+// reference's order of operations - norm first - by orders of magnitude.  It stays a launch of its own.)
 enum Epilogue : int32_t {
     EPI_RELU = 0,        // C = max(P, 0)
     EPI_GATED_GELU = 1,  // C = gelu_tanh(P0) * P1
@@ -160,12 +162,9 @@ struct GemmProblem {
     float* C;          // [rows][N]
     int N, K;
     int epilogue;
-    // EPI_RELU / EPI_GATED_GELU with the norm carried along: row_stats [rows][2] = (mu, rstd) per row of A, and
-    // for the centered form colsum [N] (colsum1 for B1) - in grouped launches those of expert 0, the others
-    // follow at weight_stride like B.  All null: the plain product.
+    // EPI_RELU / EPI_GATED_GELU with the RMS norm carried along: row_stats [rows][2] = (-, rstd) per row of A
+    // (the pairs launch_row_stats writes).  Null: the plain product.
     const float* row_stats;
-    const float* colsum;
-    const float* colsum1;
     // grouped launches only: null, or [E] where expert e's weights are at B + expert_slot[e] * weight_stride
     // instead of B + e * weight_stride (experts held in slots in whatever order they arrived)
     const int* expert_slot;

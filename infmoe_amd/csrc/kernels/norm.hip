@@ -88,47 +88,34 @@ __global__ __launch_bounds__(kThreads) void row_norm_kernel(float* __restrict__ 
     }
 }
 
-// One wave per weight row: the row times gamma, in place, and the sum of the scaled row (in float64: it is
-// subtracted from a product of the same size in the centered form).
+// One wave per weight row: the row times gamma, in place.
 template <bool VEC>
-__global__ __launch_bounds__(kThreads) void fold_gamma_kernel(float* __restrict__ w, float* __restrict__ colsum,
-                                                              const float* __restrict__ gamma, int n_rows, int d) {
+__global__ __launch_bounds__(kThreads) void fold_gamma_kernel(float* __restrict__ w, const float* __restrict__ gamma,
+                                                              int n_rows, int d) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (n >= n_rows) return;
     float* row = w + (size_t)n * d;
-    double sum = 0.0;
     if (VEC) {
         const int n4 = d >> 2;
         v4f* r4 = reinterpret_cast<v4f*>(row);
         const v4f* g4 = reinterpret_cast<const v4f*>(gamma);
-        for (int k = lane; k < n4; k += 64) {
-            const v4f v = r4[k] * g4[k];
-            r4[k] = v;
-            sum += ((double)v.x + (double)v.y) + ((double)v.z + (double)v.w);
-        }
+        for (int k = lane; k < n4; k += 64) r4[k] = r4[k] * g4[k];
     } else {
-        for (int k = lane; k < d; k += 64) {
-            const float v = row[k] * gamma[k];
-            row[k] = v;
-            sum += (double)v;
-        }
+        for (int k = lane; k < d; k += 64) row[k] = row[k] * gamma[k];
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-    if (lane == 0) colsum[n] = (float)sum;
 }
 
 }  // namespace
 
-hipError_t launch_fold_gamma(float* w, float* colsum, const float* gamma, int n_rows, int d, hipStream_t stream) {
+hipError_t launch_fold_gamma(float* w, const float* gamma, int n_rows, int d, hipStream_t stream) {
     if (n_rows <= 0) return hipSuccess;
     const dim3 grid((n_rows + kThreads / 64 - 1) / (kThreads / 64));
     const bool aligned = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gamma)) & 15) == 0;
     if (d % 4 == 0 && aligned)
-        fold_gamma_kernel<true><<<grid, kThreads, 0, stream>>>(w, colsum, gamma, n_rows, d);
+        fold_gamma_kernel<true><<<grid, kThreads, 0, stream>>>(w, gamma, n_rows, d);
     else
-        fold_gamma_kernel<false><<<grid, kThreads, 0, stream>>>(w, colsum, gamma, n_rows, d);
+        fold_gamma_kernel<false><<<grid, kThreads, 0, stream>>>(w, gamma, n_rows, d);
     return hipGetLastError();
 }
 

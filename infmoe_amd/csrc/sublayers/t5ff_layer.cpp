@@ -32,14 +32,13 @@ size_t T5FFLayer::workspaceBytes(int rows, int d, int h) {
     return sizeof(float) * (size_t)rows * ((size_t)d + (size_t)h);  // normed rows, hidden rows
 }
 
-// A device slot holds the expert's arrays in the reference's order and, behind them, the column sums of the
-// input-side matrices after gamma has been multiplied into them (one or two arrays of h floats).
-size_t T5FFLayer::weightSize() {
-    return weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind) + sizeof(float) * (size_t)(nMatrices() - 1) * mHiddenSize;
-}
+size_t T5FFLayer::weightSize() { return weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind); }
 
-// In a layer: hidden rows, then room for (mu, rstd, -, -) per row, used when nobody hands the statistics over.
-size_t T5FFLayer::layerWorkspaceBytes(int rows) const { return sizeof(float) * (size_t)rows * ((size_t)mHiddenSize + 4); }
+// Norm carried on the first product: hidden rows, then room for (-, rstd, -, -) per row, used when nobody hands
+// the statistics over.  Norm as a launch of its own: normed rows, hidden rows.
+size_t T5FFLayer::layerWorkspaceBytes(int rows) const {
+    return folds() ? sizeof(float) * (size_t)rows * ((size_t)mHiddenSize + 4) : workspaceBytes(rows, mEmbeddingSize, mHiddenSize);
+}
 
 size_t T5FFLayer::workspaceSize(int32_t tokenCount) { return align_up(layerWorkspaceBytes(tokenCount)); }
 
@@ -84,8 +83,8 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
     mVersion.fetch_add(1, std::memory_order_acq_rel);
     if (mDeviceWeights != nullptr) {
-        // already resident: the device slot is made anew from the host store, because gamma is multiplied into
-        // the input-side matrices there and either may be the array that changed (blocking; not a hot path)
+        // already resident: the device slot is made anew from the host store, because gamma may be multiplied
+        // into the input-side matrices there and either may be the array that changed (blocking; not a hot path)
         INFMOE_HIP(hipDeviceSynchronize());
         INFMOE_TRY(copyWeights(static_cast<char*>(mDeviceWeights) + deviceStride() * (size_t)expert, expert, nullptr));
         INFMOE_HIP(hipStreamSynchronize(nullptr));
@@ -171,19 +170,18 @@ Status T5FFLayer::makeResident() {
 
 Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
     // plugin/sublayers/T5FFLayer.cc:55-88 issues four copies; the host store is already packed in slot order,
-    // so one copy moves the expert.  Then, on the same stream, the norm's gamma is multiplied into the
-    // input-side matrices where they now lie and their column sums are put behind the arrays: the first
-    // product of the expert then carries the norm with it (a read and a write of those matrices in device
-    // memory, a few percent of what the copy over the host link takes).
+    // so one copy moves the expert.  Then, with the rms norm and on the same stream, the norm's gamma is
+    // multiplied into the input-side matrices where they now lie: the first product of the expert then carries
+    // the norm with it (a read and a write of those matrices in device memory, a few percent of what the copy
+    // over the host link takes).
     if (mHostWeights == nullptr) return fail(INFMOE_ERR_STATE, "T5_FF: copyWeights before initialize");
     const char* src = reinterpret_cast<const char*>(mHostWeights) + hostStride() * (size_t)expert;
     const int d = mEmbeddingSize, h = mHiddenSize;
     INFMOE_HIP(hipMemcpyAsync(dst, src, weightBytes(d, h, mFfnKind), hipMemcpyHostToDevice, stream));
+    if (!folds()) return INFMOE_OK;
     float* w = static_cast<float*>(dst);
     const size_t dh = (size_t)d * h;
-    float* colsum = w + d + (size_t)nMatrices() * dh;
-    for (int m = 0; m < nMatrices() - 1; ++m)
-        INFMOE_HIP(launch_fold_gamma(w + d + m * dh, colsum + (size_t)m * h, w, h, d, stream));
+    for (int m = 0; m < nMatrices() - 1; ++m) INFMOE_HIP(launch_fold_gamma(w + d + m * dh, w, h, d, stream));
     return INFMOE_OK;
 }
 
@@ -196,10 +194,10 @@ int T5FFLayer::skinnyMaxRows(int32_t tokenCount) const {
     return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kSkinnyMaxRows : 0;
 }
 
-// folded: `weights` is a slot as copyWeights leaves it (gamma multiplied into the input-side matrices, column
-// sums behind the arrays), the workspace is the in-layer one, and the norm rides on the first product; rowStats
-// are the rows' (mu, rstd) or null to compute them here.  Not folded: `weights` holds the arrays as the caller
-// made them (plugin/sublayers/T5FFLayer.cc:100-131), the norm is a launch of its own into the workspace.
+// folded (rms norm only): `weights` is a slot as copyWeights leaves it (gamma multiplied into the input-side
+// matrices), the workspace is [H | statistics], and the norm rides on the first product; rowStats are the rows'
+// (-, rstd) or null to compute them here.  Not folded: `weights` holds the arrays as they were given
+// (plugin/sublayers/T5FFLayer.cc:100-131), the norm is a launch of its own into the workspace [LN | H].
 Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int h, int normKind, int ffnKind,
                          const void* weights, const float* in, float* out, void* workspace, hipStream_t stream,
                          bool folded, const float* rowStats) {
@@ -217,10 +215,6 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
             rowStats = stats;
         }
         g1.A = in, g1.row_stats = rowStats;
-        if (normKind == NORM_CENTERED) {  // the rms form has no mean to take out
-            g1.colsum = w + d + (size_t)nMat * dh;
-            g1.colsum1 = ffnKind == FFN_GATED_GELU ? g1.colsum + h : nullptr;
-        }
     } else {
         float* ln = static_cast<float*>(workspace);
         hid = ln + (size_t)rows * d;
@@ -252,13 +246,13 @@ Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input
     // outside a layer call the expert stands alone: a call of tokenCount tokens over one expert, on a slot
     // that copyWeights filled
     return runOne(tokenCount, tokenCount, 1, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
-                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, true, nullptr);
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, folds(), nullptr);
 }
 
 Status T5FFLayer::runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input,
                              void* output, void* workspace, hipStream_t stream, const float* rowStats) {
     return runOne(tokenCount, layerTokens, mExpertCount, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
-                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, true, rowStats);
+                  static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, folds(), rowStats);
 }
 
 Status T5FFLayer::runGrouped(const GroupedRun& g) {
@@ -268,20 +262,24 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     const float* w = static_cast<const float*>(g.weights ? g.weights : mDeviceWeights);
     const int* slot = g.weights ? g.expertSlot : nullptr;
     float* hid = static_cast<float*>(g.workspace);
-    const float* stats = g.rowStats;
-    if (stats == nullptr) {  // a caller that did not compute them with the scatter
-        float* own = hid + (size_t)T * h;
-        INFMOE_HIP(launch_row_stats(own, g.input, T, d, mNormKind, g.stream));
-        stats = own;
-    }
     GemmProblem g1{};
     g1.expert_slot = slot;
-    g1.A = g.input, g1.row_stats = stats, g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
-    g1.B1 = mFfnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
-    if (mNormKind == NORM_CENTERED) {  // the rms form has no mean to take out
-        g1.colsum = w + d + (size_t)nMatrices() * dh;
-        g1.colsum1 = mFfnKind == FFN_GATED_GELU ? g1.colsum + h : nullptr;
+    if (folds()) {
+        const float* stats = g.rowStats;
+        if (stats == nullptr) {  // a caller that did not compute them with the scatter
+            float* own = hid + (size_t)T * h;
+            INFMOE_HIP(launch_row_stats(own, g.input, T, d, mNormKind, g.stream));
+            stats = own;
+        }
+        g1.A = g.input, g1.row_stats = stats;
+    } else {  // every routed row with the gamma of its own expert (plugin/sublayers/T5FFLayer.cc:99-103)
+        float* ln = hid;
+        hid = ln + (size_t)T * d;
+        INFMOE_HIP(launch_row_norm(ln, g.input, T, d, w, stride, g.rowExpert, mNormKind, g.stream, slot));
+        g1.A = ln;
     }
+    g1.B = w + d, g1.C = hid, g1.N = h, g1.K = d;
+    g1.B1 = mFfnKind == FFN_GATED_GELU ? w + d + dh : nullptr;
     g1.epilogue = mFfnKind == FFN_GATED_GELU ? EPI_GATED_GELU : EPI_RELU;
     GemmProblem g2{};
     g2.expert_slot = slot;

@@ -8,12 +8,14 @@
 //         "relu" with wi, wo (the dense_relu_dense the layer is named after).
 // Device slot of one expert, as plugin/sublayers/T5FFLayer.cc:100,112,118-119,130-131:
 //   [gamma d | wi h*d | wo d*h]  or  [gamma d | wi_0 h*d | wi_1 h*d | wo d*h]   (floats)
-// As copyWeights leaves it, gamma is multiplied into the input-side matrices and their column sums follow the
-// arrays: the norm then rides on the first product (rstd_r * (x.w' - mu_r * colsum)) and is no launch of its own.
-// Workspace for M rows in a layer: [H M*h | row statistics M*4] (the reference keeps the normed rows M*d and two
-// M*h buffers; here the gelu*mul product is formed in the epilogue, so one hidden buffer is all; the statistics
-// area is used when nobody hands them over).  infmoe_t5ff_run, which takes the arrays as the caller made them,
-// runs the norm as a launch of its own into [LN M*d | H M*h].
+// With the rms norm, copyWeights leaves the input-side matrices multiplied by gamma: the norm then rides on the
+// first product (rstd_r * x.w') and is no launch of its own.  Workspace for M rows: [H M*h | row statistics M*4]
+// (the reference keeps the normed rows M*d and two M*h buffers; here the gelu*mul product is formed in the
+// epilogue, so one hidden buffer is all; the statistics area is used when nobody hands them over).
+// With the centered norm the slot holds the arrays as they are and the norm runs first, as a launch of its own,
+// as in the reference: carried on the product it would subtract mu_r * (column sum of w') from x.w', two numbers
+// that are large against their difference whenever a row's mean is large against its deviation.  Workspace
+// [LN M*d | H M*h].  infmoe_t5ff_run, which takes the arrays as the caller made them, does the same for both norms.
 #pragma once
 
 #include <atomic>
@@ -39,7 +41,7 @@ class T5FFLayer : public MoESubLayer {
                hipStream_t stream) override;
     Status runInLayer(int32_t layerTokens, int32_t tokenCount, const void* weights, const void* input, void* output,
                       void* workspace, hipStream_t stream, const float* rowStats) override;
-    int rowStatsKind() const override { return mNormKind; }
+    int rowStatsKind() const override { return folds() ? NORM_RMS : NORM_NONE; }
     Status initialize() override;
     void terminate() override;
 
@@ -62,10 +64,9 @@ class T5FFLayer : public MoESubLayer {
    private:
     int mNormKind, mFfnKind;
     int nMatrices() const { return mFfnKind == FFN_GATED_GELU ? 3 : 2; }
+    bool folds() const { return mNormKind == NORM_RMS; }  // the norm rides on the first product
     size_t hostStride() const { return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind)); }
-    size_t deviceStride() const {
-        return align_up(weightBytes(mEmbeddingSize, mHiddenSize, mFfnKind) + sizeof(float) * (size_t)(nMatrices() - 1) * mHiddenSize);
-    }
+    size_t deviceStride() const { return hostStride(); }
     size_t layerWorkspaceBytes(int rows) const;
     int keyIndex(const char* key, size_t* offsetFloats, size_t* countFloats) const;
     Status ensureHostStore();

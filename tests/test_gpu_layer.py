@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def make_layer(T_shape, E, d, h, mc, variant, sublayer="T5_FF", norm="rms", ffn="relu", seed=0, bias=None,
-               weight_file=""):
+               weight_file="", tweak=None):
     B, S = T_shape
     x, c, g = O.draw_inputs(seed, B * S, d, E)
     cfg = MoELayerConfig(seq_len=S, expert_count=E, embedding_size=d, hidden_size=h, max_concurrency=mc,
@@ -23,6 +23,8 @@ def make_layer(T_shape, E, d, h, mc, variant, sublayer="T5_FF", norm="rms", ffn=
     ws = None
     if sublayer == "T5_FF":
         ws = [O.draw_expert(seed, e, d, h, ffn) for e in range(E)]
+        if tweak is not None:
+            tweak(x, ws)
         if not weight_file:
             for e, w in enumerate(ws):
                 for k, v in w.items():
@@ -114,6 +116,28 @@ def test_variants_streamed_and_resident(torch_cuda, variant, norm, ffn, mc):
     shape, E, d, h = (4, 100), 6, 128, 384
     plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, variant, norm=norm, ffn=ffn, seed=5)
     run_and_check(torch_cuda, plugin, x, c, g, ws, shape, variant, norm=norm, ffn=ffn)
+    plugin.terminate()
+
+
+@pytest.mark.parametrize("shape", [(4, 128), (1, 24)])  # matrix-core tiles; few-row kernel
+@pytest.mark.parametrize("norm", ["centered", "rms"])
+def test_rows_with_a_large_mean_and_weights_with_a_common_sign(torch_cuda, shape, norm):
+    """The expert norm is applied after the first product, as rstd * (x W'^T - mean * colsum(W')).  With a row
+    mean of several standard deviations and weights that all have one sign, x W'^T and mean * colsum are both
+    hundreds of times larger than their difference: the case in which that order of operations loses most.
+    The layer still has to meet the float64 oracle, which norms first, to the usual bound."""
+    E, d, h = 4, 2048, 512
+
+    def tweak(x, ws):
+        rng = np.random.default_rng(77)
+        x += rng.uniform(-4, 4, size=(x.shape[0], 1)).astype(np.float32)  # per-row mean of up to 4 sigma
+        for w in ws:
+            for k in w:
+                if k.startswith("wi"):
+                    w[k] += np.float32(2.0 / np.sqrt(d))  # two standard deviations of the entries: nearly all positive
+
+    plugin, x, c, g, ws = make_layer(shape, E, d, h, E, "default", norm=norm, seed=23, tweak=tweak)
+    run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "default", norm=norm)
     plugin.terminate()
 
 

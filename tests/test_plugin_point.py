@@ -25,10 +25,10 @@ def toy():
     return lib
 
 
-def toy_config(E, d, mc, variant, B, S, seed=5):
+def toy_config(E, d, mc, variant, B, S, seed=5, kind="ToyAffine"):
     x, c, g = O.draw_inputs(seed, B * S, d, E)
     cfg = MoELayerConfig(seq_len=S, expert_count=E, embedding_size=d, hidden_size=16, max_concurrency=mc,
-                         moe_variant=variant, sublayer_type="ToyAffine", max_batch_size=B, expert_centroids=c,
+                         moe_variant=variant, sublayer_type=kind, max_batch_size=B, expert_centroids=c,
                          layernorm_weight=g if variant == "cpm_2" else None)
     return cfg, x, c, g
 
@@ -68,4 +68,25 @@ def test_out_of_tree_expert_runs_on_both_schedules(toy, torch_cuda, variant, mc)
         a = O.sigmoid(coeff)[:, None]
         post = a * post + (1 - a) * x
     np.testing.assert_allclose(y, post, rtol=2e-6, atol=1e-6)
+    plugin.terminate()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d", [48, 1024, 130])  # rows in registers, 16 bytes at a time; the same, longer; scalar path
+def test_expert_type_that_asks_for_row_statistics(toy, torch_cuda, d):
+    """A sub-layer whose rowStatsKind() is the centered norm gets (mean, 1/sqrt(biased variance + 1e-6)) of each of
+    its rows from the layer's scatter, here with means far from zero."""
+    torch = torch_cuda
+    E, B, S = 5, 2, 33
+    cfg, x, c, g = toy_config(E, d, E, "default", B, S, seed=9, kind="ToyStandardize")
+    x = (x + np.random.default_rng(1).uniform(-5, 5, size=(B * S, 1))).astype(np.float32)
+    plugin = MoELayerPlugin(cfg).create_plugin()
+    plugin.configure([B, S, d])
+    plugin.initialize()
+    y = plugin.forward(torch.from_numpy(x.reshape(B, S, d)).cuda())
+    torch.cuda.synchronize()
+    y = y.cpu().numpy().reshape(B * S, d)
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-6)
+    np.testing.assert_allclose(y, want, rtol=1e-5, atol=2e-6)
     plugin.terminate()
