@@ -80,7 +80,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 // beforehand, and the product becomes rstd_r * acc before the activation, which is the product of the
 // normed rows with the plain weights (stats: [row][2], of which [1] = rstd_r is used).  The inner loop does
 // not know of any of it.
-template <int NMB, int G4, int BN, int EPI, int BK>
+// D: register sets of the global loads, i.e. how many K steps they run ahead of the matrix core (2 or 4).
+template <int NMB, int G4, int BN, int EPI, int BK, int D>
 __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const float* __restrict__ R,
                                           float* __restrict__ C, int rows, const float* __restrict__ B0,
                                           const float* __restrict__ B1, int n0, int N, int K,
@@ -140,9 +141,15 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     for (int p = 0; p < B_LOADS; ++p)
         b_off[p] = ((unsigned)min((p / KH) * 32 + ld_row, N - 1 - n0) * (unsigned)K + 32u * (p % KH) + 4u * ld_c4) * 4u;
 
-    // Two register sets: global loads run two K steps ahead of the matrix core, which covers the
-    // latency of an HBM miss (every weight load is one) with two steps of MFMA work.
-    v4f ra[2][A_LOADS], rb[2][NB][B_LOADS];
+    // D register sets: global loads run D K steps ahead of the matrix core.  Two steps of MFMA work cover the
+    // latency of an HBM miss (every weight load is one) when a tile has a hundred rows or more.  A tile of a few
+    // dozen rows has little arithmetic per step; near the point where the weights' arrival and the arithmetic
+    // take equally long (about 40 rows) a wait for a load stalls the matrix core, and four sets take 2-3 % off
+    // calls with 50-77 rows per expert.  (For taller tiles they cost more registers than they save waits: with
+    // four sets up to 128 rows the same calls ran 3 % slower.  Where the weights alone set the pace, below 32
+    // rows, the depth makes no difference.)
+    static_assert(D == 2 || D == 4, "the step loop is unrolled by D");
+    v4f ra[D][A_LOADS], rb[D][NB][B_LOADS];
     // item L of the global loads of the step starting at k0 (K % BK == 0 on this path), into set P
     auto gload = [&](auto setc, auto lc, int k0) {
         constexpr int P = decltype(setc)::value, L = decltype(lc)::value;
@@ -150,7 +157,10 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             ra[P][L] = *reinterpret_cast<const v4f*>(a_base + (size_t)k0 * 4 + a_off[L]);
         } else {
             constexpr int M = (L - A_LOADS) / B_LOADS, Q = (L - A_LOADS) % B_LOADS;
-            rb[P][M][Q] = *reinterpret_cast<const v4f*>(b_base[M] + (size_t)k0 * 4 + b_off[Q]);
+            // a weight byte is read by one workgroup, once (by a few where an expert has several row tiles):
+            // streamed past the caches.  With few rows per expert, where the weights' arrival sets the pace, that
+            // is worth 3-6 % (256-512 tokens over 32 experts); with many it changes nothing.
+            rb[P][M][Q] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(b_base[M] + (size_t)k0 * 4 + b_off[Q]));
         }
     };
     // item L of register set P into LDS buffer BUF
@@ -195,20 +205,23 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
 
     // One K step = S slots.  A slot issues a few memory operations and then a handful of MFMAs,
     // and nothing may be moved across a slot boundary, so the matrix core is fed continuously:
-    //   * the first half of the slots carries the global loads of step s + 2 (register set 1 - P),
-    //   * the second half writes register set P (step s + 1) into LDS buffer 1 - P,
-    //   * every slot group carries the LDS operand reads of the next k group.
-    // The loop over steps is unrolled by two so that P, and with it every LDS address offset and
+    //   * the first half of the slots carries the global loads of step s + D, into register set s % D (whose
+    //     previous content, step s, went to LDS during step s - 1),
+    //   * the second half writes register set (s + 1) % D (step s + 1) into LDS buffer (s + 1) % 2,
+    //   * every slot group carries the LDS operand reads of the next k group (from LDS buffer s % 2).
+    // The loop over steps is unrolled by D so that P = s % D, and with it every LDS address offset and
     // register index, is a compile-time constant.
     constexpr int G32 = BK / 8, G16 = BK / 16;  // k groups of a step
     constexpr int S32 = N32 > 0 ? 4 * G32 : 0, S16 = T16 ? 4 * G16 : 0, S = S32 + S16, SV = S / 2;
     constexpr int R32 = NB + N32 + G4, R16 = 1 + 2 * NB;
     const int nk = K / BK;
-    auto step = [&](auto setc, int s) {
-        constexpr int P = decltype(setc)::value;
-        const std::integral_constant<int, P> cur{};
-        const std::integral_constant<int, 1 - P> other{};
-        const int kload = min(s + 2, nk - 1) * BK;  // the surplus loads of the last two steps are discarded
+    auto step = [&](auto pc, int s) {
+        constexpr int P = decltype(pc)::value;
+        const std::integral_constant<int, P % 2> cur{};          // LDS buffer the matrix core reads
+        const std::integral_constant<int, 1 - P % 2> other{};    // LDS buffer being filled
+        const std::integral_constant<int, P> lset{};             // register set being loaded
+        const std::integral_constant<int, (P + 1) % D> sset{};   // register set written to LDS
+        const int kload = min(s + D, nk - 1) * BK;  // the surplus loads of the last D steps are discarded
         if constexpr (N32 > 0)
             static_for<0, R32>([&](auto qc) { read32(cur, std::integral_constant<int, 0>{}, qc); });
         else
@@ -216,10 +229,10 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         static_for<0, S>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
             if constexpr (t < SV)
-                static_for<(t * NV) / SV, ((t + 1) * NV) / SV>([&](auto lc) { gload(other, lc, kload); });
+                static_for<(t * NV) / SV, ((t + 1) * NV) / SV>([&](auto lc) { gload(lset, lc, kload); });
             else
                 static_for<((t - SV) * NV) / (S - SV), ((t - SV + 1) * NV) / (S - SV)>(
-                    [&](auto lc) { lstore(cur, lc, other); });
+                    [&](auto lc) { lstore(sset, lc, other); });
             if constexpr (t < S32) {
                 constexpr int g = t / 4, j = t % 4;
                 if constexpr (g < G32 - 1 && j < 3)  // a third of the next group's operands per slot
@@ -256,16 +269,18 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         });
         __syncthreads();
     };
-    const std::integral_constant<int, 0> set0{};
-    const std::integral_constant<int, 1> set1{};
-    static_for<0, NV>([&](auto lc) { gload(set1, lc, 0); });
-    static_for<0, NV>([&](auto lc) { lstore(set1, lc, set0); });
-    static_for<0, NV>([&](auto lc) { gload(set0, lc, min(1, nk - 1) * BK); });
+    // step 0 into set 0 and on into LDS buffer 0, steps 1 .. D-1 into their sets
+    const std::integral_constant<int, 0> zero{};
+    static_for<0, NV>([&](auto lc) { gload(zero, lc, 0); });
+    static_for<1, D>([&](auto jc) {
+        static_for<0, NV>([&](auto lc) { gload(jc, lc, min((int)decltype(jc)::value, nk - 1) * BK); });
+    });
+    static_for<0, NV>([&](auto lc) { lstore(zero, lc, zero); });
     __syncthreads();
-    for (int s = 0; s < nk; s += 2) {
-        step(set0, s);
-        if (s + 1 < nk) step(set1, s + 1);
-    }
+    for (int s = 0; s < nk; s += D)
+        static_for<0, D>([&](auto pc) {
+            if (s + decltype(pc)::value < nk) step(pc, s + decltype(pc)::value);
+        });
 
     // epilogue
     // 32x32 block: register r holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
@@ -395,6 +410,10 @@ __device__ __forceinline__ TileShape tile_shape(int rows, bool wide) {
     return groups;
 }
 
+// Register sets of the global loads (gemm_tile's D) for a tile of 16 * nmb + 4 * g4 rows: tiles of up to 64
+// rows keep four steps in flight, taller ones two.
+constexpr int depth_of(int nmb, int g4) { return 16 * nmb + 4 * g4 <= 64 ? 4 : 2; }
+
 template <int BN, int EPI>
 __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, float* C, int rows, const float* B0,
                                               const float* B1, int n0, int N, int K, const float* stats,
@@ -411,13 +430,14 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
         if constexpr ((n) <= kMaxMb && ((g) == 0 || (!GATED && (n) >= 2 && (n) < kMaxMb))) {                    \
             if constexpr (!GATED && 16 * (n) + 4 * (g) <= 16 * kMaxMb64) {                                      \
                 if (wide) {                                                                                     \
-                    gemm_tile<n, g, BN, EPI, 64>(A, R, C, rows, B0, B1, n0, N, K, stats, smem,                  \
-                                                 min(a_alloc_rows, 16 * kMaxMb64));                             \
+                    gemm_tile<n, g, BN, EPI, 64, depth_of(n, g)>(A, R, C, rows, B0, B1, n0, N, K, stats, smem,  \
+                                                                 min(a_alloc_rows, 16 * kMaxMb64));             \
                     break;                                                                                      \
                 }                                                                                               \
             }                                                                                                   \
             if constexpr ((g) == 0 || 16 * (n) + 4 * (g) > 16 * kMaxMb64)                                       \
-                gemm_tile<n, g, BN, EPI, 32>(A, R, C, rows, B0, B1, n0, N, K, stats, smem, a_alloc_rows);       \
+                gemm_tile<n, g, BN, EPI, 32, depth_of(n, g)>(A, R, C, rows, B0, B1, n0, N, K, stats, smem,      \
+                                                             a_alloc_rows);                                     \
         }                                                                                                       \
         break;
 #define INFMOE_CASE(n) INFMOE_CASE_G(n, 0) INFMOE_CASE_G(n, 1) INFMOE_CASE_G(n, 2)
