@@ -317,9 +317,9 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     int T = 0;
     INFMOE_TRY(checkDims(dims, nbDims, &T));
     if (!mInitialized) return fail(INFMOE_ERR_STATE, "enqueue before initialize");
+    if (T == 0) return INFMOE_OK;  // an empty batch has nothing to read or write: its tensors may have no memory at all
     if (inputs == nullptr || outputs == nullptr || inputs[0] == nullptr || outputs[0] == nullptr)
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "null input or output");
-    if (T == 0) return INFMOE_OK;
     // An earlier call met a token without an orderable score (a NaN in its row) and the device has said so
     // since: reported once, by the first call that sees it; this call queues nothing.
     if (*static_cast<volatile int32_t*>(mNanFlagHost) != 0) {

@@ -304,6 +304,31 @@ def test_near_tie_tokens_are_compared_under_either_expert(torch_cuda, variant):
     plugin.terminate()
 
 
+@pytest.mark.parametrize("mc", [2, 6])  # experts streamed / resident
+@pytest.mark.parametrize("variant", ["cpm_2", "base_layer"])
+def test_batch_size_may_change_from_call_to_call(torch_cuda, variant, mc):
+    """The batch dimension is dynamic (the reference takes it from the input descriptor of every enqueue,
+    plugin/MoELayerPlugin.cc:284-289): one handle, one workspace sized for the largest batch, calls of 4, 1, 0, 3
+    and 4 sequences, each against the oracle on its own tokens."""
+    torch = torch_cuda
+    S, E, d, h = 40, 6, 128, 256
+    plugin, x, c, g, ws = make_layer((4, S), E, d, h, mc, variant, seed=31)
+    x3 = x.reshape(4, S, d)
+    for B in (4, 1, 0, 3, 4):
+        y = plugin.forward(dev(torch, x3[:B]))
+        torch.cuda.synchronize()
+        assert tuple(y.shape) == (B, S, d)
+        if B == 0:
+            continue
+        xb = x3[:B].reshape(B * S, d)
+        ref = O.moe_layer(xb, c, variant, ws, layernorm_weight=g)
+        assert (O.top2_relative_gap(ref["aff"]) >= 1e-6).all()
+        count, stats = plugin.last_routing()
+        np.testing.assert_array_equal(count, ref["count"])
+        assert_close(y.cpu().numpy().reshape(B * S, d), ref["out"], what=f"batch of {B}")
+    plugin.terminate()
+
+
 def test_single_token(torch_cuda):
     shape, E, d, h = (1, 1), 4, 64, 128
     for mc in (2, 4):
