@@ -81,6 +81,7 @@ struct GateArgs {
     int* nan_flag;    // null, or an int (host memory the device can write) set to 1 when a token has no orderable score
     float* partials;  // [slices][T][E + 2]: dot products, row sum, row sum of squares
     float* gpart;     // [groups][slices][2E]: sum and sum of squares of the folded centroid slice
+    int* zero_stats;  // GATE_SLICES only: null, or the 4 ints the later combine launch counts into, set to zero here
 };
 
 // Four floats of a row starting at k.  With VEC (d % 4 == 0, 16-byte aligned rows) the load is
@@ -153,6 +154,8 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg)
     const int g = mode == GATE_SLICES ? blockIdx.x / S : blockIdx.x;
     const int j = mode == GATE_SLICES ? blockIdx.x % S : 0;
     const int t0 = g * TM;
+    // the routing statistics the combine launch counts into start at zero (saves a fill launch)
+    if (mode == GATE_SLICES && arg.zero_stats != nullptr && blockIdx.x == 0 && tid < 4) arg.zero_stats[tid] = 0;
 
     if (tid < TM) {
         s_best[tid] = -FLT_MAX;  // plugin/cuda/moe.cu:26-27
@@ -909,8 +912,12 @@ hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* ce
     } else {
         plan = gate_plan(T, d, E, vec, partial_floats);
         if (zero_stats && stats != nullptr) {
-            const hipError_t err = launch_fill_i32(stats, 4, 0, stream);
-            if (err != hipSuccess) return err;
+            if (plan.slices > 1) {  // two launches: the first clears what the second counts into
+                a.zero_stats = stats;
+            } else {
+                const hipError_t err = launch_fill_i32(stats, 4, 0, stream);
+                if (err != hipSuccess) return err;
+            }
         }
     }
     a.gpart = scratch ? scratch + (size_t)plan.slices * T * (E + 2) : nullptr;

@@ -75,10 +75,13 @@ __global__ __launch_bounds__(64 * WAVES) void gate_slab_kernel(const float* __re
     const int my_tiles = first_tile >= all_tiles ? 0 : min(tiles_per_wave, (all_tiles - first_tile + WAVES - 1) / WAVES);
     const int total = my_tiles * nch;
 
-    // register sets of 8 KB per wave: chunk n sits in set n % SETS, and SETS - 1 chunks are in flight while one
-    // is consumed.  Two sets: with four (three at 64 experts), which the registers would allow, the launch
-    // took a fifth longer (4096 tokens x 4096 x 32 experts: 23.2 us against 19.1; 16384 x 2048 x 64: 53.6
-    // against 47.7) - the matrix work of a wave then starts only when most of its loads have landed.
+    // Register sets of 8 KB per wave: chunk n sits in set n % SETS, and SETS - 1 chunks are in flight while one
+    // is consumed.  Two sets.  More, which the registers would allow, make the launch slower, not faster (4096
+    // tokens x 4096 x 32 experts: 19.1 us with two, 21.0 with three, 23.3 with four; 16384 x 2048 x 64: 49.5 /
+    // 54.1 / 55.3), also with the slab's loads issued ahead of the tokens' so that they are not waited for
+    // together.  The launch is not short of bytes in flight: between 2048 and 4096 tokens of 4096 floats it
+    // takes 5.5 us more for 33.6 MB more (6.1 TB/s); the rest, 8 us, is what a launch, the slab's fill and the
+    // last tiles' stores cost once.  (Non-temporal loads of the tokens change nothing.)
     constexpr int SETS = 2;
     v4f xa[SETS][kGroupsPerChunk];
     int ltile = first_tile, lchunk = 0;  // load cursor
@@ -93,14 +96,11 @@ __global__ __launch_bounds__(64 * WAVES) void gate_slab_kernel(const float* __re
             ltile += WAVES;
         }
     };
-    // the first SETS - 1 chunks go out before the slab is filled
-    static_for_sets<0, SETS - 1>([&](auto uc) {
-        if (decltype(uc)::value < total) load_into(uc);
-    });
-
     {   // slice j of every centroid row -> LDS (rows beyond E are zero: their columns are never stored).
-        // ks is a power of two times 128, so (row, float4) of item idx are a shift and a mask; the loop is
-        // unrolled so that eight loads per thread are in flight before the first is stored.
+        // ks is a power of two times 128, so (row, float4) of item idx are a shift and a mask; every pass has eight
+        // loads per thread in flight before the first is stored.  The wave's first SETS - 1 chunks of tokens go out
+        // between the loads and the stores of the last pass: loads complete in the order they were issued, so the
+        // slab's are waited for alone, with the tokens' still on their way.
         const int n4 = ks / 4, sh = 31 - __clz(n4);
         const int items = EP * n4;
 #pragma unroll 1
@@ -111,6 +111,12 @@ __global__ __launch_bounds__(64 * WAVES) void gate_slab_kernel(const float* __re
                 const int idx = min(base + u * 64 * WAVES + tid, items - 1);
                 const int e = idx >> sh, c = idx & (n4 - 1);
                 v[u] = *reinterpret_cast<const v4f*>(Cf + (size_t)min(e, E - 1) * d + k0 + 4 * c);
+            }
+            if (base + 8 * 64 * WAVES >= items) {
+                static_for_sets<0, SETS - 1>([&](auto uc) {
+                    if (decltype(uc)::value < total) load_into(uc);
+                });
+                __builtin_amdgcn_sched_barrier(0);  // the tokens' loads stay in front of the slab's stores
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
