@@ -31,11 +31,11 @@ PCIE_PEAK_GBS = 64.0           # host link, PCIe Gen5 x16, one direction
 # (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt,
 # profiles/c4_expert_gemm_grouped_kernel_stats.txt;
 # counters cannot be read from inside a run).  Kept as the ratio counter bytes / algorithmic bytes of the
-# profiled launches (c2: 5.72 GB on average over the two launches against 5.60 GB of weights and
-# activations; c5: 4.03 GB against 4.03 GB of weights of 24 active experts; c4: 7.67 GB against 4.97 GB, the
+# profiled launches (c2: 5.77 GB on average over the two launches against 5.60 GB of weights and
+# activations; c5: 4.03 GB against 4.03 GB of weights of 24 active experts; c4: 7.90 GB against 4.97 GB, the
 # weights of an expert with more than 256 rows being fetched once per row tile) and applied to the
 # algorithmic bytes of the run at hand, whose number of active experts may differ.
-MEASURED_TRAFFIC_RATIO = {"c2": 5.72 / 5.60, "c5": 4.03 / 4.03, "c4": 7.67 / 4.97}
+MEASURED_TRAFFIC_RATIO = {"c2": 5.77 / 5.60, "c5": 4.03 / 4.03, "c4": 7.90 / 4.97}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf

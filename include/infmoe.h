@@ -79,6 +79,9 @@ typedef struct infmoe_plugin infmoe_plugin; /* opaque: replaces class MoELayerPl
  *   ffn_kind   chars: "relu" (default; weights wi_weight, wo_weight) |
  *                     "gated_gelu" (weights wi_0_weight, wi_1_weight, wo_weight)
  * Arrays and strings are copied; the caller keeps ownership of `fields`.
+ * Any positive sizes are accepted, as in the reference.  The matrix-core expert kernels take embedding_size and
+ * hidden_size that are multiples of 32 (every size in the reference's examples but the README's toy one); other
+ * sizes compute the same results on a plain one-output-per-thread kernel at a few percent of that speed.
  */
 int32_t infmoe_create(const char* layer_name, const infmoe_field* fields, int32_t n_fields, infmoe_plugin** out);
 

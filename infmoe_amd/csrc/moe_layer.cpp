@@ -81,7 +81,7 @@ MoELayer::~MoELayer() { (void)terminate(); }
 Status MoELayer::setScoreBias(const float* host) {
     if (host == nullptr) {
         mScoreBias.clear();
-    } else {
+    } else if (host != mScoreBias.data()) {  // (initialize() hands the stored values back in to upload them)
         mScoreBias.assign(host, host + mParams.expertCount);
     }
     if (mInitialized) {
