@@ -366,6 +366,53 @@ def test_clone_shares_weights_and_serialization_round_trip(torch_cuda):
     plugin.terminate()
 
 
+@pytest.mark.parametrize("mc", [2, 4])  # experts streamed (each clone its own slots and copy stream) / resident
+def test_clones_driven_from_two_threads_at_once(torch_cuda, mc):
+    """Stacked layers share one sub-layer (plugin/MoELayerPlugin.cc:114-127).  Two clones, each called from a thread
+    of its own on a stream of its own with a batch of its own, while the other runs: every output has to be the one the
+    layer gives when nothing else is going on."""
+    import threading
+    torch = torch_cuda
+    E, d, h = 4, 128, 256
+    shapes = [(2, 60), (3, 33)]
+    plugin, x0, c, g, ws = make_layer(shapes[0], E, d, h, mc, "cpm_2", seed=57)
+    twin = plugin.clone()
+    twin.configure([shapes[1][0], shapes[1][1], d])
+    twin.initialize()
+    x1 = O.draw_inputs(58, shapes[1][0] * shapes[1][1], d, E)[0]
+    layers = [plugin, twin]
+    xs = [dev(torch, x0.reshape(*shapes[0], d)), dev(torch, x1.reshape(*shapes[1], d))]
+    want = [layers[i].forward(xs[i]).clone() for i in range(2)]
+    torch.cuda.synchronize()
+    for i, x in enumerate((x0, x1)):
+        ref = O.moe_layer(x, c, "cpm_2", ws, layernorm_weight=g)
+        assert_close(want[i].cpu().numpy().reshape(-1, d), ref["out"], what=f"clone {i} alone")
+    errors = []
+
+    def drive(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    y = layers[i].forward(xs[i])
+                    stream.synchronize()
+                    if not torch.equal(y, want[i]):
+                        errors.append(f"clone {i}: output differs")
+                        return
+        except Exception as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append(f"clone {i}: {exc!r}")
+
+    threads = [threading.Thread(target=drive, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a thread did not finish"
+    assert not errors, errors
+    twin.terminate()
+    plugin.terminate()
+
+
 def save_experts(path, ws, compressed=False):
     arrays = {f"{e}/{k}": v for e, w in enumerate(ws) for k, v in w.items()}
     (np.savez_compressed if compressed else np.savez)(path, **arrays)
