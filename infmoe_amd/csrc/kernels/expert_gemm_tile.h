@@ -207,12 +207,17 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     // and nothing may be moved across a slot boundary, so the matrix core is fed continuously:
     //   * the first half of the slots carries the global loads of step s + D, into register set s % D (whose
     //     previous content, step s, went to LDS during step s - 1),
-    //   * the second half writes register set (s + 1) % D (step s + 1) into LDS buffer (s + 1) % 2,
-    //   * every slot group carries the LDS operand reads of the next k group (from LDS buffer s % 2).
+    //   * the second half, but for its last two slots, writes register set (s + 1) % D (step s + 1) into LDS
+    //     buffer (s + 1) % 2; then the workgroup's one barrier of the step,
+    //   * every slot group carries the LDS operand reads of the next k group (from LDS buffer s % 2), and the
+    //     last two slots, behind the barrier, those of the first k group of step s + 1 from the buffer just
+    //     filled: the next step's first matrix instructions find their operands there instead of waiting for
+    //     them at the top of the step with nothing else to do (worth 1 % on calls with 50-77 rows per expert,
+    //     nothing on tall tiles: the wait was shorter than it looks in the source).
     // The loop over steps is unrolled by D so that P = s % D, and with it every LDS address offset and
     // register index, is a compile-time constant.
     constexpr int G32 = BK / 8, G16 = BK / 16;  // k groups of a step
-    constexpr int S32 = N32 > 0 ? 4 * G32 : 0, S16 = T16 ? 4 * G16 : 0, S = S32 + S16, SV = S / 2;
+    constexpr int S32 = N32 > 0 ? 4 * G32 : 0, S16 = T16 ? 4 * G16 : 0, S = S32 + S16, SV = S / 2, SB = S - 2;
     constexpr int R32 = NB + N32 + G4, R16 = 1 + 2 * NB;
     const int nk = K / BK;
     auto step = [&](auto pc, int s) {
@@ -222,17 +227,26 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         const std::integral_constant<int, P> lset{};             // register set being loaded
         const std::integral_constant<int, (P + 1) % D> sset{};   // register set written to LDS
         const int kload = min(s + D, nk - 1) * BK;  // the surplus loads of the last D steps are discarded
-        if constexpr (N32 > 0)
-            static_for<0, R32>([&](auto qc) { read32(cur, std::integral_constant<int, 0>{}, qc); });
-        else
-            static_for<0, R16>([&](auto qc) { read16(cur, std::integral_constant<int, 0>{}, qc); });
         static_for<0, S>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
-            if constexpr (t < SV)
+            if constexpr (t < SV) {
                 static_for<(t * NV) / SV, ((t + 1) * NV) / SV>([&](auto lc) { gload(lset, lc, kload); });
-            else
-                static_for<((t - SV) * NV) / (S - SV), ((t - SV + 1) * NV) / (S - SV)>(
+            } else if constexpr (t < SB) {
+                static_for<((t - SV) * NV) / (SB - SV), ((t - SV + 1) * NV) / (SB - SV)>(
                     [&](auto lc) { lstore(sset, lc, other); });
+            } else {
+                // every wave's share of step s + 1 is in LDS; nobody reads buffer `cur` any more (the last k
+                // group's operands were waited for two slots ago)
+                if constexpr (t == SB) __syncthreads();
+                if constexpr (N32 > 0)
+                    static_for<0, R32>([&](auto qc) {
+                        if constexpr (decltype(qc)::value % 2 == t - SB) read32(other, std::integral_constant<int, 0>{}, qc);
+                    });
+                else
+                    static_for<0, R16>([&](auto qc) {
+                        if constexpr (decltype(qc)::value % 2 == t - SB) read16(other, std::integral_constant<int, 0>{}, qc);
+                    });
+            }
             if constexpr (t < S32) {
                 constexpr int g = t / 4, j = t % 4;
                 if constexpr (g < G32 - 1 && j < 3)  // a third of the next group's operands per slot
@@ -267,7 +281,6 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             }
             __builtin_amdgcn_sched_barrier(0);
         });
-        __syncthreads();
     };
     // step 0 into set 0 and on into LDS buffer 0, steps 1 .. D-1 into their sets
     const std::integral_constant<int, 0> zero{};
@@ -277,6 +290,11 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     });
     static_for<0, NV>([&](auto lc) { lstore(zero, lc, zero); });
     __syncthreads();
+    // the first step's first operands (every later step's are read in the last slots of the step before)
+    if constexpr (N32 > 0)
+        static_for<0, R32>([&](auto qc) { read32(zero, zero, qc); });
+    else
+        static_for<0, R16>([&](auto qc) { read16(zero, zero, qc); });
     for (int s = 0; s < nk; s += D)
         static_for<0, D>([&](auto pc) {
             if (s + decltype(pc)::value < nk) step(pc, s + decltype(pc)::value);
