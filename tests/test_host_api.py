@@ -216,3 +216,26 @@ def test_generated_weight_file_has_reference_key_names(tmp_path):
         assert set(z.files) == {f"{e}/{k}" for e in range(2)
                                 for k in ("layer_norm_weight", "wi_0_weight", "wi_1_weight", "wo_weight")}  # README.md:121
         assert z["0/wi_0_weight"].shape == (8, 4) and z["1/wo_weight"].shape == (4, 8)
+
+
+def test_header_is_plain_c_and_usable_without_hip_headers(tmp_path):
+    """include/infmoe.h compiles as C99 (-pedantic, no HIP or C++ headers on the include path) and a C program
+    linked against libinfmoe.so drives the host side of the life cycle: tests/c_abi/use_from_c.c."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    assert gcc is not None, "gcc is needed for this test"
+    capi.load()  # fails loudly when the library has not been built
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib_dir = os.path.join(root, "infmoe_amd", "lib")
+    exe = str(tmp_path / "use_from_c")
+    r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I" + os.path.join(root, "include"),
+                        os.path.join(root, "tests", "c_abi", "use_from_c.c"), "-L" + lib_dir, "-linfmoe",
+                        "-Wl,-rpath," + lib_dir, "-o", exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    first, second = r.stdout.strip().splitlines()
+    assert first.startswith("name=MoELayerPlugin version=1 workspace=")
+    assert f"bad_dims_status={capi.ERR_INVALID_ARGUMENT} " in first and "expected embedding_size = 64" in first
+    assert second == f"bad_variant_status={capi.ERR_UNSUPPORTED}"
