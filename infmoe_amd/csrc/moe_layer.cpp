@@ -634,13 +634,14 @@ Status MoELayer::serialize(void* buffer, size_t bytes) const {
     char* p = static_cast<char*>(buffer) + sizeof(head);
     char* s = p;
     for (const std::string* str : {&mParams.weightFile, &mParams.sublayerType, &mParams.variant}) {
-        memcpy(s, str->data(), str->size());
+        if (!str->empty()) memcpy(s, str->data(), str->size());
         s += str->size();
     }
     p += align_up((size_t)(s - p), 4);
-    memcpy(p, mParams.centroids.data(), 4 * mParams.centroids.size());
+    // (an empty vector's data() may be null, which memcpy must not be given even for no bytes)
+    if (!mParams.centroids.empty()) memcpy(p, mParams.centroids.data(), 4 * mParams.centroids.size());
     p += 4 * mParams.centroids.size();
-    memcpy(p, mParams.layernormWeight.data(), 4 * mParams.layernormWeight.size());
+    if (!mParams.layernormWeight.empty()) memcpy(p, mParams.layernormWeight.data(), 4 * mParams.layernormWeight.size());
     return INFMOE_OK;
 }
 
@@ -662,9 +663,9 @@ Status MoELayer::deserialize(const char* layerName, const void* data, size_t byt
     p.variant.assign(s + l1 + l2, l3);
     const char* f = s + align_up(l1 + l2 + l3, 4);
     p.centroids.resize(nc);
-    memcpy(p.centroids.data(), f, 4 * nc);
+    if (nc > 0) memcpy(p.centroids.data(), f, 4 * nc);
     p.layernormWeight.resize(nl);
-    memcpy(p.layernormWeight.data(), f + 4 * nc, 4 * nl);
+    if (nl > 0) memcpy(p.layernormWeight.data(), f + 4 * nc, 4 * nl);
     const uint32_t storedFlags = head[8];
     INFMOE_TRY(create(std::move(p), out));
     // the flags are a function of the variant string (plugin/MoELayerPlugin.cc:44-58); a blob whose flag
