@@ -122,7 +122,11 @@ int32_t infmoe_initialize(infmoe_plugin* p);
  * Replaces MoELayerPlugin::enqueue (plugin/MoELayerPlugin.cc:279-416).
  * inputs[0]: device float [B,S,d]; outputs[0]: device float [B,S,d]; `workspace`: device,
  * at least infmoe_workspace_size bytes, 256-byte aligned; `hip_stream`: hipStream_t.
- * Allocates no device memory (the streamed schedule builds a short list of experts on the host heap).
+ * Allocates nothing, neither device nor host memory, on either schedule (the lists the streamed schedule makes
+ * per call live in the layer, sized by infmoe_initialize).
+ *
+ * Streams: the weight slots of a streamed layer (max_concurrency < expert_count) keep experts between calls, so a
+ * call on another stream than the previous call's first waits, on the device, for that call's end.
  *
  * A token whose scores cannot be ordered (a NaN in its row; the reference asserts there,
  * plugin/cuda/moe.cu:70,184) does not stop the call, whatever the schedule: the call completes, that
@@ -130,8 +134,12 @@ int32_t infmoe_initialize(infmoe_plugin* p);
  * in stats[1] of infmoe_last_routing.  INFMOE_ERR_NAN is returned once per such call, by whichever
  * of these comes first: the call itself when it waits for the routing anyway (experts streamed,
  * max_concurrency < expert_count); the first later infmoe_enqueue on the handle that finds the
- * device's report (that call returns the code and queues nothing); not at all if infmoe_last_routing
- * has reported the count in between.
+ * device's report - a DEFERRED NOTICE: that later call is queued in full, its own output is valid, and
+ * the message (infmoe_last_error) names the number of the call that met the NaN (calls that queue work
+ * are counted from 1 per handle since infmoe_initialize); not at all if infmoe_last_routing has reported
+ * the count in between.  The host looks for the report only inside infmoe_enqueue: a caller that
+ * replays a captured graph of the layer never enters it and has to poll infmoe_last_routing (stats[1])
+ * if it wants to know.
  */
 int32_t infmoe_enqueue(infmoe_plugin* p, const int32_t* dims, int32_t nb_dims, const void* const* inputs,
                        void* const* outputs, void* workspace, void* hip_stream);

@@ -45,11 +45,12 @@ DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-pa
 
 
 def _newest_header() -> float:
-    newest = os.path.getmtime(os.path.join(HERE, "..", "include", "infmoe.h"))
-    for root, _, files in os.walk(CSRC):
-        for f in files:
-            if f.endswith(".h"):
-                newest = max(newest, os.path.getmtime(os.path.join(root, f)))
+    newest = 0.0
+    for top in (os.path.join(HERE, "..", "include"), CSRC):  # the public headers are included by the sources too
+        for root, _, files in os.walk(top):
+            for f in files:
+                if f.endswith(".h"):
+                    newest = max(newest, os.path.getmtime(os.path.join(root, f)))
     return newest
 
 

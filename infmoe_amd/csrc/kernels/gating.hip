@@ -78,7 +78,8 @@ struct GateArgs {
     int mode;       // GateMode
     int slices;     // workgroups per token group
     int steps_per;  // K chunks per slice
-    int* nan_flag;    // null, or an int (host memory the device can write) set to 1 when a token has no orderable score
+    int* nan_flag;    // null, or an int (host memory the device can write) set to nan_value when a token has no orderable score
+    int nan_value;
     float* partials;  // [slices][T][E + 2]: dot products, row sum, row sum of squares
     float* gpart;     // [groups][slices][2E]: sum and sum of squares of the folded centroid slice
     int* zero_stats;  // GATE_SLICES only: null, or the 4 ints the later combine launch counts into, set to zero here
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg)
                 sel[t] = 0;
                 coeff[t] = __builtin_nanf("");  // marks the row: the combine step writes NaN for it
                 if (stats) atomicAdd(&stats[1], 1);
-                if (arg.nan_flag) *reinterpret_cast<volatile int*>(arg.nan_flag) = 1;
+                if (arg.nan_flag) *reinterpret_cast<volatile int*>(arg.nan_flag) = arg.nan_value;
             } else {
                 sel[t] = I;
                 coeff[t] = B;
@@ -871,7 +872,7 @@ size_t gate_scratch_floats(int T, int d, int E) {
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids, const float* centroid_stats,
-                            float* scratch, size_t scratch_floats, bool zero_stats, int* nan_flag) {
+                            float* scratch, size_t scratch_floats, bool zero_stats, int* nan_flag, int nan_value) {
     if (T <= 0) return zero_stats && stats ? launch_fill_i32(stats, 4, 0, stream) : hipSuccess;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(centroids) |
                            reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(folded_centroids)) & 15) == 0;
@@ -895,7 +896,7 @@ hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* ce
     a.T = T, a.d = d, a.E = E;
     a.X = x, a.C = centroids, a.gamma = gamma, a.Cf = folded_centroids, a.cstats = centroid_stats;
     a.norm_kind = norm_kind, a.bias = score_bias, a.sel = sel, a.coeff = coeff, a.stats = stats;
-    a.nan_flag = nan_flag;
+    a.nan_flag = nan_flag, a.nan_value = nan_value;
     a.partials = scratch;
     GatePlan plan{};
     GateSlabPlan slab{};
@@ -935,7 +936,7 @@ hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* ce
     }
     if (err != hipSuccess || !lean) return err;
     return launch_gate_combine(T, d, E, plan.slices, scratch, centroid_stats, x, centroids, use_gamma ? gamma : nullptr,
-                               norm_kind, score_bias, sel, coeff, stats, nan_flag, stream);
+                               norm_kind, score_bias, sel, coeff, stats, nan_flag, stream, nan_value);
 }
 
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats) {

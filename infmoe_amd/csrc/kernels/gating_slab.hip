@@ -224,7 +224,8 @@ struct CombineArgs {
     int* sel;
     float* coeff;
     int* stats;     // or null
-    int* nan_flag;  // null, or an int (host memory the device can write) set to 1 when a token has no orderable score
+    int* nan_flag;  // null, or an int (host memory the device can write) set to nan_value when a token has no orderable score
+    int nan_value;
 };
 
 __device__ __forceinline__ double wave_sum64(double v) {
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
         a.coeff[t] = besti < 0 ? __builtin_nanf("") : best;  // NaN marks the row: the combine step writes NaN for it
         if (besti < 0) {
             if (a.stats != nullptr) atomicAdd(&a.stats[1], 1);
-            if (a.nan_flag != nullptr) *reinterpret_cast<volatile int*>(a.nan_flag) = 1;
+            if (a.nan_flag != nullptr) *reinterpret_cast<volatile int*>(a.nan_flag) = a.nan_value;
         }
     }
 
@@ -508,10 +509,20 @@ bool gate_slab_plan(int T, int d, int E, size_t scratch_floats, GateSlabPlan* pl
     return true;
 }
 
+// Enough for every call of up to T tokens, not only for one of exactly T: the plan cuts d into MORE slices when
+// there are fewer tokens (until tiles * slices reaches 8 * 256), so slices(T') * T' is not monotone in T', and a
+// caller sizes one workspace for its largest batch and then calls with any smaller one.  slices(T') never grows
+// with T', so the largest product on [1, T] sits at the right end of a stretch of constant slice count: at T
+// itself or at the last token count before some slice count s makes the plan stop, 16 * (ceil(8 * 256 / s) - 1).
 size_t gate_slab_scratch_floats(int T, int d, int E) {
-    GateSlabPlan p{};
-    if (!gate_slab_plan(T, d, E, (size_t)-1, &p)) return 0;
-    return (size_t)p.slices * T * ((size_t)E + 2);
+    size_t most = 0;
+    auto at = [&](int t) {
+        GateSlabPlan p{};
+        if (t >= 1 && t <= T && gate_slab_plan(t, d, E, (size_t)-1, &p)) most = std::max(most, (size_t)p.slices * t);
+    };
+    at(T);
+    for (int s = 2; s <= kGateMaxSlices; ++s) at(16 * ((8 * 256 + s - 1) / s - 1));
+    return most * ((size_t)E + 2);
 }
 
 hipError_t launch_gate_slab(const GateSlabPlan& p, int T, int d, int E, const float* x, const float* folded_centroids,
@@ -544,13 +555,13 @@ bool gate_combine_ok(int d, int E) { return E <= 128 && d % 4 == 0; }
 hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* partials, const float* centroid_stats,
                                const float* x, const float* centroids, const float* gamma, int norm_kind,
                                const float* score_bias, int* sel, float* coeff, int* stats, int* nan_flag,
-                               hipStream_t stream) {
+                               hipStream_t stream, int nan_value) {
     if (T <= 0) return hipSuccess;
     if (!gate_combine_ok(d, E) || slices < 1 || slices > kGateMaxSlices) return hipErrorInvalidValue;
     CombineArgs a{};
     a.T = T, a.d = d, a.E = E, a.S = slices;
     a.partials = partials, a.cstats = centroid_stats, a.X = x, a.C = centroids, a.gamma = gamma, a.bias = score_bias;
-    a.norm_kind = norm_kind, a.sel = sel, a.coeff = coeff, a.stats = stats, a.nan_flag = nan_flag;
+    a.norm_kind = norm_kind, a.sel = sel, a.coeff = coeff, a.stats = stats, a.nan_flag = nan_flag, a.nan_value = nan_value;
     const dim3 grid((T + 15) / 16);
     switch (nblk_of(E)) {
         case 1: gate_combine_kernel<1><<<grid, 256, 0, stream>>>(a); break;

@@ -30,13 +30,14 @@ constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/subla
 // launches where there are two, else by a small fill launch; without it the caller has cleared them.
 // A token without an orderable score (a NaN in its row; the reference asserts, plugin/cuda/moe.cu:70) gets
 // expert 0 and the coefficient NaN, is counted in stats[1], and sets *nan_flag (an int the device can
-// write, e.g. page-locked host memory) to 1 when that pointer is given.
+// write, e.g. page-locked host memory) to nan_value (say, a number that names the call) when that pointer is given.
 size_t gate_scratch_floats(int T, int d, int E);
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids = nullptr,
                             const float* centroid_stats = nullptr, float* scratch = nullptr,
-                            size_t scratch_floats = 0, bool zero_stats = false, int* nan_flag = nullptr);
+                            size_t scratch_floats = 0, bool zero_stats = false, int* nan_flag = nullptr,
+                            int nan_value = 1);
 // Calls with many tokens: the first of two launches writes partial scores per slice of the embedding
 // dimension with that slice of the folded centroids resident in LDS (gating_slab.hip); the combine launch
 // of the gating kernel adds the slices and selects.  The plan says how a call is cut; gate_slab_plan
@@ -65,7 +66,7 @@ bool gate_combine_ok(int d, int E);
 hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* partials, const float* centroid_stats,
                                const float* x, const float* centroids, const float* gamma, int norm_kind,
                                const float* score_bias, int* sel, float* coeff, int* stats, int* nan_flag,
-                               hipStream_t stream);
+                               hipStream_t stream, int nan_value = 1);
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)

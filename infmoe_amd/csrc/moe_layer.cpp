@@ -3,6 +3,8 @@
 #include <sys/stat.h>
 
 #include <algorithm>
+#include <atomic>
+#include <cstdio>
 #include <cstring>
 
 namespace infmoe {
@@ -195,10 +197,12 @@ Status MoELayer::initialize() {
     return s;
 }
 
-// The launch geometry of the kernels is fixed for the part they are written for: workgroup ids are dealt
+// The launch geometry of the kernels is tuned for the part they are written for: workgroup ids are dealt
 // round-robin to 8 accelerator dies (the row-tile schedule of the grouped expert launch and the slice map of
-// the gating count on it) and one workgroup per compute unit means 256 of them.  A device partitioned
-// differently would still compute the same results but balance badly, so it is refused, loudly.
+// the gating count on it) and one workgroup per compute unit means 256 of them.  No result depends on it: every
+// workgroup finds its work from its id alone, whichever die runs it.  A device partitioned differently (an
+// MI355X in CPX/DPX mode, another gfx950 part) computes the same bits with a worse balance, so it is told
+// once per process, on stderr, and served.
 static Status check_device_geometry() {
     int dev = 0, cus = 0, xccs = 0;
     INFMOE_HIP(hipGetDevice(&dev));
@@ -207,10 +211,12 @@ static Status check_device_geometry() {
         (void)hipGetLastError();
         xccs = kXcdCount;  // a runtime that cannot tell: the compute-unit count decides
     }
-    if (cus != 256 || xccs != kXcdCount)
-        return fail(INFMOE_ERR_UNSUPPORTED,
-                    "device %d has %d compute units in %d accelerator dies; this library schedules for 256 in %d (an MI355X in "
-                    "its single-partition mode)", dev, cus, xccs, kXcdCount);
+    static std::atomic<bool> told{false};
+    if ((cus != 256 || xccs != kXcdCount) && !told.exchange(true))
+        fprintf(stderr,
+                "infmoe: device %d has %d compute units in %d accelerator dies; the launch schedules are tuned for 256 in %d "
+                "(an MI355X in its single-partition mode): results are the same, the load balance is not\n",
+                dev, cus, xccs, kXcdCount);
     return INFMOE_OK;
 }
 
@@ -265,7 +271,13 @@ Status MoELayer::initializeSteps() {
         for (auto& e : mCopyDone) INFMOE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
         for (auto& e : mComputeDone) INFMOE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
         INFMOE_HIP(hipEventCreateWithFlags(&mFork, hipEventDisableTiming));
+        INFMOE_HIP(hipEventCreateWithFlags(&mCallDone, hipEventDisableTiming));
+        mHaveCallDone = false, mLastStream = nullptr;
+        for (auto* v : {&mNeeded, &mOrder, &mSlotOf, &mSlotTableSent}) v->reserve(E);
+        mStreamSlots.reserve(2 * (size_t)mParams.maxConcurrency);
+        mLastUse.reserve(mParams.maxConcurrency);
     }
+    mCallNumber = 0;
     mInitialized = true;
     if (!mScoreBias.empty()) INFMOE_TRY(setScoreBias(mScoreBias.data()));
     return INFMOE_OK;
@@ -305,7 +317,9 @@ Status MoELayer::terminate() {
     mTimingDepth = 0;
     if (mFork) (void)hipEventDestroy(mFork);
     if (mRoutingDone) (void)hipEventDestroy(mRoutingDone);
-    mFork = mRoutingDone = nullptr;
+    if (mCallDone) (void)hipEventDestroy(mCallDone);
+    mFork = mRoutingDone = mCallDone = nullptr;
+    mHaveCallDone = false, mLastStream = nullptr;
     mInitialized = false;
     return INFMOE_OK;
 }
@@ -320,15 +334,14 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     if (T == 0) return INFMOE_OK;  // an empty batch has nothing to read or write: its tensors may have no memory at all
     if (inputs == nullptr || outputs == nullptr || inputs[0] == nullptr || outputs[0] == nullptr)
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "null input or output");
-    // An earlier call met a token without an orderable score (a NaN in its row) and the device has said so
-    // since: reported once, by the first call that sees it; this call queues nothing.
-    if (*static_cast<volatile int32_t*>(mNanFlagHost) != 0) {
-        *static_cast<volatile int32_t*>(mNanFlagHost) = 0;
-        return fail(INFMOE_ERR_NAN, "an earlier infmoe_enqueue on this layer met token(s) with no orderable score (NaN input?); "
-                                    "their output rows are NaN");
-    }
     if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255))
         return fail(INFMOE_ERR_INVALID_ARGUMENT, "workspace must be non-null and 256-byte aligned");
+    // An earlier call met a token without an orderable score (a NaN in its row) and the device has said so
+    // since, by writing that call's number into the flag.  It is reported once, by the first call that sees it:
+    // a deferred notice.  The present call is queued in full all the same, and its own output is not touched by
+    // the notice.
+    const int32_t earlierNan = __atomic_exchange_n(mNanFlagHost, 0, __ATOMIC_ACQ_REL);
+    mCallNumber = mCallNumber == 0x7fffffff ? 1 : mCallNumber + 1;
     const int E = mParams.expertCount, d = mParams.embeddingSize;
     const float* x = static_cast<const float*>(inputs[0]);
     float* y = static_cast<float*>(outputs[0]);
@@ -350,7 +363,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
                                 mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream, mFoldedGpu,
                                 mFoldedGpu + (size_t)E * d, c.gateScratch, gate_scratch_floats(T, d, E),
-                                /*zero_stats=*/true, mNanFlagDev));
+                                /*zero_stats=*/true, mNanFlagDev, mCallNumber));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     // (the row tiles of the grouped expert launch are made on either schedule: streamed experts that are all
@@ -394,10 +407,20 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream, c.routedCoeff));
     INFMOE_TRY(mark(7));
     if (timed) ++mTimedCalls;
-    if (!grouped && mNanRowsSeen > 0) {
-        *static_cast<volatile int32_t*>(mNanFlagHost) = 0;  // reported here, not again by the next call
-        return fail(INFMOE_ERR_NAN, "%d token(s) have no orderable score (NaN input?); their output rows are NaN", mNanRowsSeen);
+    if (!grouped) {
+        INFMOE_HIP(hipEventRecord(mCallDone, stream));
+        mHaveCallDone = true, mLastStream = stream;
     }
+    if (!grouped && mNanRowsSeen > 0) {
+        // reported here, not again by the next call (the routing was waited for, so the flag is this call's)
+        __atomic_store_n(mNanFlagHost, 0, __ATOMIC_RELEASE);
+        return fail(INFMOE_ERR_NAN, "%d token(s) of this call (number %d on this layer) have no orderable score (NaN input?); "
+                                    "their output rows are NaN", mNanRowsSeen, mCallNumber);
+    }
+    if (earlierNan != 0)
+        return fail(INFMOE_ERR_NAN, "call number %d on this layer met token(s) with no orderable score (NaN input?) and wrote "
+                                    "NaN output rows for them; this call (number %d) was queued in full and is not affected",
+                    earlierNan, mCallNumber);
     return INFMOE_OK;
 }
 
@@ -471,6 +494,9 @@ Status MoELayer::lastTiming(float* ms) {
 Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedRun& g) {
     const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
     const size_t routingInts = (size_t)2 * E + 1 + 4;
+    // The slots outlive the call.  Work of an earlier call that reads or fills them was joined into THAT call's
+    // stream; a call on another stream waits for its end before it touches a slot.
+    if (mHaveCallDone && stream != mLastStream) INFMOE_HIP(hipStreamWaitEvent(stream, mCallDone, 0));
     INFMOE_HIP(hipMemcpyAsync(mRoutingHost, mRoutingGpu, sizeof(int32_t) * routingInts, hipMemcpyDeviceToHost, stream));
     INFMOE_HIP(hipStreamSynchronize(stream));
     const int32_t* count = mRoutingHost;
@@ -488,17 +514,24 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedR
     // index; here the ones with most rows go first (stable, so equal counts stay ascending): every
     // expert costs the same copy, and the compute that nothing can hide is the last expert's, so it
     // should be the shortest.  Rows of different experts are disjoint: the order cannot change a bit.
-    std::vector<int> needed;
-    needed.reserve(E);
+    // (the lists are members with room reserved in initialize(): nothing here touches the heap)
+    std::vector<int>&needed = mNeeded, &order = mOrder, &slotOf = mSlotOf, &streamSlots = mStreamSlots, &lastUse = mLastUse;
+    needed.clear();
     for (int e = 0; e < E; ++e)
         if (count[e] > 0) needed.push_back(e);
-    std::stable_sort(needed.begin(), needed.end(), [&](int a, int b) { return count[a] > count[b]; });
-    std::vector<int> slotOf(E, -1);
+    // (an insertion sort: stable, in place - std::stable_sort takes a temporary buffer from the heap - and E is small)
+    for (size_t i = 1; i < needed.size(); ++i) {
+        const int e = needed[i];
+        size_t j = i;
+        for (; j > 0 && count[needed[j - 1]] < count[e]; --j) needed[j] = needed[j - 1];
+        needed[j] = e;
+    }
+    slotOf.assign(E, -1);
     for (int s = 0; s < mc; ++s)
         if (mSlotExpert[s] >= 0) slotOf[mSlotExpert[s]] = s;
     // Experts still in a slot run first, from there and without a copy; the others follow, most rows first,
     // through the slots that are not retained.
-    std::vector<int> order;
+    order.clear();
     for (const int e : needed)
         if (slotOf[e] >= 0) order.push_back(e);
     const int present = (int)order.size(), absent = (int)needed.size() - present;
@@ -510,7 +543,7 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedR
     // Slots the absent experts pass through, in the order they become free: first those that hold nothing
     // this call needs, then those of the experts that run from them once more and are then given up (in the
     // order they run).  Slot numbers break ties, so the choice is deterministic.
-    std::vector<int> streamSlots;
+    streamSlots.clear();
     for (int s = 0; s < mc; ++s)
         if (mSlotExpert[s] < 0 || count[mSlotExpert[s]] == 0) streamSlots.push_back(s);
     for (int k = keep; k < present; ++k) streamSlots.push_back(slotOf[order[k]]);
@@ -530,7 +563,7 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedR
     INFMOE_HIP(hipEventRecord(mFork, stream));
     INFMOE_HIP(hipStreamWaitEvent(mCopyStream, mFork, 0));
     for (auto s : mComputeStreams) INFMOE_HIP(hipStreamWaitEvent(s, mFork, 0));
-    std::vector<int> lastUse(mc, -1);  // position in `order` of the expert that last ran from the slot in this call
+    lastUse.assign(mc, -1);  // position in `order` of the expert that last ran from the slot in this call
     // Whatever happens in the loop, the compute streams forked above are joined back into the caller's
     // stream before returning: an error half way must not leave work that nothing waits for.
     auto queueExperts = [&]() -> Status {
@@ -564,18 +597,23 @@ Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedR
         return INFMOE_OK;
     };
     const Status queued = queueExperts();
-    const std::string why = queued != INFMOE_OK ? last_error_slot() : std::string();
-    // the copy stream's last work is waited for by a compute stream unless the loop broke off in between
-    if (queued != INFMOE_OK) {
-        INFMOE_HIP(hipEventRecord(mFork, mCopyStream));
-        INFMOE_HIP(hipStreamWaitEvent(stream, mFork, 0));
-    }
-    for (size_t i = 0; i < mComputeStreams.size(); ++i) {
-        INFMOE_HIP(hipEventRecord(mJoin[i], mComputeStreams[i]));
-        INFMOE_HIP(hipStreamWaitEvent(stream, mJoin[i], 0));
-    }
-    if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, stream));
-    if (queued != INFMOE_OK) last_error_slot() = why;
+    auto join = [&]() -> Status {
+        // the copy stream's last work is waited for by a compute stream unless the loop broke off in between
+        if (queued != INFMOE_OK) {
+            INFMOE_HIP(hipEventRecord(mFork, mCopyStream));
+            INFMOE_HIP(hipStreamWaitEvent(stream, mFork, 0));
+        }
+        for (size_t i = 0; i < mComputeStreams.size(); ++i) {
+            INFMOE_HIP(hipEventRecord(mJoin[i], mComputeStreams[i]));
+            INFMOE_HIP(hipStreamWaitEvent(stream, mJoin[i], 0));
+        }
+        if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, stream));
+        return INFMOE_OK;
+    };
+    if (queued == INFMOE_OK) return join();
+    const std::string why = last_error_slot();  // (the error path only: the message of the first failure is the one kept)
+    (void)join();
+    last_error_slot() = why;
     return queued;
 }
 

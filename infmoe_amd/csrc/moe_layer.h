@@ -81,6 +81,7 @@ class MoELayer {
     int32_t* mNanFlagHost = nullptr;  // in the same allocation: set by the gating kernels, read by the host
     int32_t* mNanFlagDev = nullptr;   // its device address
     int mNanRowsSeen = 0;             // streamed schedule: NaN rows of the call in progress
+    int32_t mCallNumber = 0;          // calls that queued work, 1-based; what the device writes into the NaN flag
     char* mSlotPool = nullptr;        // streamed experts: max_concurrency weight slots, kept between calls
     std::vector<int> mSlotExpert;     // expert held by each slot, -1 for none
     int32_t* mSlotTableGpu = nullptr;   // [E] slot of every expert, for launches over all experts from the slots
@@ -92,6 +93,14 @@ class MoELayer {
     std::vector<hipStream_t> mComputeStreams;
     std::vector<hipEvent_t> mCopyDone, mComputeDone, mJoin;
     hipEvent_t mFork = nullptr, mRoutingDone = nullptr;
+    // streamed schedule: the slots are state that outlives a call, so a call on another stream than the last one's
+    // first waits for that one's end
+    hipEvent_t mCallDone = nullptr;
+    hipStream_t mLastStream = nullptr;
+    bool mHaveCallDone = false;
+    // streamed schedule: lists made per call, with room for E (or max_concurrency) entries from initialize() on, so
+    // that a call touches no allocator
+    std::vector<int> mNeeded, mOrder, mSlotOf, mStreamSlots, mLastUse;
     bool mTiming = false;
     int mTimingDepth = 0;            // calls whose marks are kept
     long long mTimedCalls = 0;       // timed calls since timing was switched on

@@ -78,6 +78,11 @@ Status T5FFLayer::setWeights(int expert, const char* key, const float* host, siz
     // the reference asserts on the byte count of every array (plugin/sublayers/T5FFLayer.cc:62,69,76,83)
     if (count != cnt) return fail(INFMOE_ERR_INVALID_ARGUMENT, "%s: expected %zu floats, got %zu", key, cnt, count);
     INFMOE_TRY(ensureHostStore());
+    if (mCopiesQueued.exchange(false, std::memory_order_acq_rel)) {
+        // streamed experts: a copy out of the host store that an earlier call queued may still be on its way,
+        // and must not read half of the old and half of the new array (blocking; not a hot path)
+        INFMOE_HIP(hipDeviceSynchronize());
+    }
     float* slot = reinterpret_cast<float*>(reinterpret_cast<char*>(mHostWeights) + hostStride() * (size_t)expert);
     memcpy(slot + off, host, cnt * sizeof(float));
     mHave[(size_t)expert * (nMatrices() + 1) + idx] = 1;
@@ -178,6 +183,7 @@ Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
     const char* src = reinterpret_cast<const char*>(mHostWeights) + hostStride() * (size_t)expert;
     const int d = mEmbeddingSize, h = mHiddenSize;
     INFMOE_HIP(hipMemcpyAsync(dst, src, weightBytes(d, h, mFfnKind), hipMemcpyHostToDevice, stream));
+    mCopiesQueued.store(true, std::memory_order_release);
     if (!folds()) return INFMOE_OK;
     float* w = static_cast<float*>(dst);
     const size_t dh = (size_t)d * h;

@@ -76,6 +76,7 @@ class T5FFLayer : public MoESubLayer {
     std::vector<uint8_t> mHave;      // [E][nMatrices+1] which arrays have been provided
     void* mDeviceWeights = nullptr;  // E slots when resident
     std::atomic<uint64_t> mVersion{0};  // bumped by every setWeights
+    std::atomic<bool> mCopiesQueued{false};  // a copy out of the host store may be in flight
 };
 
 }  // namespace infmoe

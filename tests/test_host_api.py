@@ -239,3 +239,32 @@ def test_header_is_plain_c_and_usable_without_hip_headers(tmp_path):
     assert first.startswith("name=MoELayerPlugin version=1 workspace=")
     assert f"bad_dims_status={capi.ERR_INVALID_ARGUMENT} " in first and "expected embedding_size = 64" in first
     assert second == f"bad_variant_status={capi.ERR_UNSUPPORTED}"
+
+
+@pytest.mark.parametrize("E,d,h,variant,tmax", [
+    (32, 4096, 10240, "cpm_2", 9000),     # the headline layer: the gating cuts d into more slices for fewer tokens
+    (64, 2048, 8192, "base_layer", 18000),
+    (4, 64, 256, "default", 3000),
+    (128, 1024, 512, "default", 5000),
+    (7, 384, 96, "cpm_2", 3000),
+])
+def test_workspace_size_never_shrinks_as_tokens_grow(E, d, h, variant, tmax):
+    """A caller sizes ONE workspace for its largest batch (getWorkspaceSize, plugin/MoELayerPlugin.cc:253-273) and
+    then calls with any smaller batch; enqueue lays the blocks out from the call's own token count, so the size has
+    to be non-decreasing in the token count or a smaller batch would be laid out past the end of the buffer."""
+    lib = capi.load()
+    kw = dict(expert_count=E, embedding_size=d, hidden_size=h, max_concurrency=E,
+              expert_centroids=np.zeros(E * d, np.float32), expert_sublayer_type="T5_FF", moe_variant=variant)
+    if variant == "cpm_2":
+        kw["layernorm_weight"] = np.ones(d, np.float32)
+    for ffn in ("relu", "gated_gelu"):
+        status, hnd, msg = create(**kw, ffn_kind=ffn)
+        assert status == capi.OK, msg
+        out = C.c_size_t()
+        prev, worst = 0, 0
+        for t in range(0, tmax + 1):
+            assert lib.infmoe_workspace_size(hnd, (C.c_int32 * 3)(1, t, d), 3, C.byref(out)) == capi.OK
+            worst = max(worst, prev - out.value)
+            prev = max(prev, out.value)
+        lib.infmoe_destroy(hnd)
+        assert worst == 0, f"a smaller batch needs up to {worst} bytes more than a larger one"
