@@ -1,18 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c5|c4|c3|c1] [--no-cpu] [--no-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c5|c4|c3|c1|ex] [--no-cpu] [--no-secondary]
 
 A step is one infmoe_enqueue over one batch of synthetic input that is already resident in
 HBM.  The default workload is the configuration the headline metric is quoted on: cpm_2,
 E=32, d=4096, h=10240, FP32, 4096 tokens, all experts resident.  One JSON line is printed:
-whole-layer tokens/s, the roofline of the dominant kernel (measured with HIP events on the
-stream the kernels run on) and the C/OpenMP restatement of the same math timed on the host
-cores on a bounded sample of the same workload.
+whole-layer tokens/s (median of the K per-step times, taken with the library's phase marks switched
+off), the roofline of the dominant kernel (from a second pass of K steps with the phase marks on: HIP
+events on the stream the kernels run on) and the C/OpenMP restatement of the same math timed on the
+host cores on a bounded sample of the same workload.  Under "secondary" the same line carries the
+other regimes of the same run: the decode shape, the streamed configuration with its overlap
+efficiency, the skewed workload with the expert kernels' rate against rows per expert, a token sweep
+between decode and prefill, and the vendor's batched FP32 GEMM on the uniform version of the same
+problem next to the library's expert launches on a uniformly routed batch.
 """
 from __future__ import annotations
 
 import argparse
+import concurrent.futures
+import hashlib
 import json
 import os
 import sys
@@ -26,16 +33,26 @@ sys.path.insert(0, ROOT)
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense FP32 matrix
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 PCIE_PEAK_GBS = 64.0           # host link, PCIe Gen5 x16, one direction
-# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
-# benchmark scaled by what the same counters read for the row-copy kernels of known size
-# (profiles/c2_expert_gemm_grouped_kernel_stats.txt, profiles/c5_expert_skinny_kernel_stats.txt,
-# profiles/c4_expert_gemm_grouped_kernel_stats.txt;
-# counters cannot be read from inside a run).  Kept as the ratio counter bytes / algorithmic bytes of the
-# profiled launches (c2: 5.77 GB on average over the two launches against 5.60 GB of weights and
-# activations; c5: 4.03 GB against 4.03 GB of weights of 24 active experts; c4: 7.90 GB against 4.97 GB, the
-# weights of an expert with more than 256 rows being fetched once per row tile) and applied to the
-# algorithmic bytes of the run at hand, whose number of active experts may differ.
-MEASURED_TRAFFIC_RATIO = {"c2": 5.77 / 5.60, "c5": 4.03 / 4.03, "c4": 7.90 / 4.97}
+# HBM bytes per launch of the dominant kernel cannot be counted from inside a run: they come from rocprofv3
+# FETCH_SIZE / WRITE_SIZE runs of this benchmark, scaled by what the same counters read for the row-copy
+# kernels of known size, and are kept as the ratio (counter bytes) / (algorithmic bytes) of the profiled
+# launches, applied to the algorithmic bytes of the run at hand (whose number of active experts may differ).
+# Each entry names the summary it was taken from and the digest of the kernel source that summary was
+# collected with; the JSON line repeats both next to the digest of the source as it is now, so that a
+# figure that has outlived its kernel shows as stale.
+KERNEL_SOURCES = {
+    "gemm": ("infmoe_amd/csrc/kernels/expert_gemm_tile.h", "infmoe_amd/csrc/kernels/expert_gemm.hip",
+             "infmoe_amd/csrc/kernels/dispatch.hip"),
+    "skinny": ("infmoe_amd/csrc/kernels/expert_skinny.hip",),
+}
+MEASURED_TRAFFIC = {
+    "c2": dict(ratio=5.77 / 5.60, kernel="gemm", source="profiles/c2_expert_gemm_grouped_kernel_stats.txt",
+               source_digest="unrecorded"),
+    "c5": dict(ratio=4.03 / 4.03, kernel="skinny", source="profiles/c5_expert_skinny_kernel_stats.txt",
+               source_digest="unrecorded"),
+    "c4": dict(ratio=7.90 / 4.97, kernel="gemm", source="profiles/c4_expert_gemm_grouped_kernel_stats.txt",
+               source_digest="unrecorded"),
+}
 
 CONFIGS = {
     # name: variant, E, d, h, mc, (B, S), zipf
@@ -48,6 +65,41 @@ CONFIGS = {
     # sub-layer, 80 x 512 tokens, experts streamed through four slots
     "ex": dict(variant="cpm_2", E=20, d=4096, h=16384, mc=4, shape=(80, 512), zipf=False, layers=3),
 }
+
+
+def source_digest(kind):
+    hsh = hashlib.sha256()
+    for rel in KERNEL_SOURCES[kind]:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            hsh.update(f.read())
+    return hsh.hexdigest()[:12]
+
+
+def traffic_of(name, algorithmic_bytes):
+    """(bytes, provenance) of the dominant kernel's HBM traffic per launch, or (None, None)."""
+    t = MEASURED_TRAFFIC.get(name)
+    if t is None:
+        return None, None
+    now = source_digest(t["kernel"])
+    return round(t["ratio"] * algorithmic_bytes), {
+        "ratio_counter_over_algorithmic": round(t["ratio"], 4), "from": t["source"],
+        "kernel_source_digest_when_profiled": t["source_digest"], "kernel_source_digest_now": now,
+        "stale": t["source_digest"] != now}
+
+
+# ---------------------------------------------------------------- synthetic tensors
+# numpy default_rng on a SeedSequence(0) child per tensor: tensors do not depend on the order they are drawn in
+# and the experts can be generated side by side.  Matrices are drawn in their logical shape (centroids [d,E],
+# wi [d,h], wo [h,d]) and handed over in the layout the layer takes them in ([E][d], [h][d], [d][h]).
+def _rng(*key):
+    return np.random.default_rng(np.random.SeedSequence(entropy=0, spawn_key=tuple(key)))
+
+
+def _normal(key, shape, scale=1.0):
+    a = _rng(*key).standard_normal(shape, dtype=np.float32)
+    if scale != 1.0:
+        a *= np.float32(scale)
+    return a
 
 
 def zipf_score_bias(x, centroids, s=1.2, iters=30):
@@ -64,57 +116,87 @@ def zipf_score_bias(x, centroids, s=1.2, iters=30):
     return bias.astype(np.float32)
 
 
-def build_layer(torch, cfg, seed=0, keep_host=True, replicate=False):
-    """Synthetic tensors drawn on the GPU (fixed seed), expert weights handed to the library by
-    host pointer, as a caller holding an npz in memory would."""
+def draw_slot(e, d, h, n_inner):
+    """Packed weights of expert e: [gamma | wi [h][d] | wo [d][h]], or [gamma | wi_0 | wi_1 | wo]."""
+    import torch  # (its blocked CPU transpose is ten times faster than numpy's strided copy)
+    slot = np.empty(d + (n_inner + 1) * d * h, np.float32)
+    slot[:d] = 1.0 + 0.1 * _normal((100 + e, 0), d)
+
+    def put(dst, logical):
+        torch.from_numpy(dst).copy_(torch.from_numpy(logical).t())
+
+    for i in range(n_inner):
+        put(slot[d + i * d * h:d + (i + 1) * d * h].reshape(h, d), _normal((100 + e, 1 + i), (d, h), d ** -0.5))
+    put(slot[d + n_inner * d * h:].reshape(d, h), _normal((100 + e, 3), (h, d), h ** -0.5))
+    return slot
+
+
+def build_layer(torch, cfg, keep_host=True, replicate=False, slots=None):
+    """Synthetic tensors (see above), uploaded once; expert weights handed to the library by host pointer, as a
+    caller holding an npz in memory would.  `slots`: packed experts drawn earlier (a second layer over the same
+    weights)."""
     from infmoe_amd import MoELayerConfig, MoELayerPlugin
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = cfg["shape"]
     T = B * S
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(seed)
-    x = torch.randn(T, d, generator=gen, device="cuda")
-    cent = (torch.randn(d, E, generator=gen, device="cuda") / d ** 0.5).t().contiguous()  # logical [d,E] -> [E][d]
-    gamma = 1 + 0.1 * torch.randn(d, generator=gen, device="cuda")
+    x = torch.from_numpy(_normal((0,), (T, d))).cuda()
+    cent_host = np.ascontiguousarray(_normal((1,), (d, E), d ** -0.5).T)  # logical [d,E] -> [E][d]
+    gamma_host = 1.0 + 0.1 * _normal((2,), d)
     gated = cfg.get("ffn", "relu") == "gated_gelu"
     mcfg = MoELayerConfig(seq_len=S, expert_count=E, embedding_size=d, hidden_size=h, max_concurrency=cfg["mc"],
                           moe_variant=cfg["variant"], sublayer_type="T5_FF", max_batch_size=B,
-                          ffn_kind=cfg.get("ffn", "relu"),
-                          expert_centroids=cent.cpu().numpy(),
-                          layernorm_weight=gamma.cpu().numpy() if cfg["variant"] == "cpm_2" else None)
+                          ffn_kind=cfg.get("ffn", "relu"), expert_centroids=cent_host,
+                          layernorm_weight=gamma_host if cfg["variant"] == "cpm_2" else None)
     plugin = MoELayerPlugin(mcfg).create_plugin()
-    slots = []
-    # [gamma | wi [h][d] | wo [d][h]], or [gamma | wi_0 | wi_1 | wo] for the gated form
     inner = ("wi_0_weight", "wi_1_weight") if gated else ("wi_weight",)
-    slot_floats = d + (len(inner) + 1) * d * h
 
-    def hand_over(e, base):
+    def hand_over(e, slot):
+        base = slot.ctypes.data
         plugin.set_expert_weights_ptr(e, "layer_norm_weight", base, d)
         for i, name in enumerate(inner):
             plugin.set_expert_weights_ptr(e, name, base + 4 * (d + i * d * h), d * h)
         plugin.set_expert_weights_ptr(e, "wo_weight", base + 4 * (d + len(inner) * d * h), d * h)
 
-    for e in range(E):
-        if replicate and e > 0:  # profiling runs: every expert gets expert 0's values (same work, short set-up)
-            hand_over(e, slots[0].ctypes.data if keep_host else slot.ctypes.data)
-            if keep_host:
-                slots.append(slots[0])
-            continue
-        slot = np.empty(slot_floats, np.float32)
-        slot[:d] = (1 + 0.1 * torch.randn(d, generator=gen, device="cuda")).cpu().numpy()
-        for i in range(len(inner)):
-            slot[d + i * d * h:d + (i + 1) * d * h] = (torch.randn(h, d, generator=gen, device="cuda") / d ** 0.5).cpu().numpy().ravel()
-        slot[d + len(inner) * d * h:] = (torch.randn(d, h, generator=gen, device="cuda") / h ** 0.5).cpu().numpy().ravel()
-        hand_over(e, slot.ctypes.data)
-        if keep_host:
-            slots.append(slot)
+    if slots is None:
+        # profiling runs: every expert gets expert 0's values (same work, short set-up)
+        todo = [0] if replicate else list(range(E))
+        workers = min(len(todo), max(1, min(16, os.cpu_count() or 1)))
+        kept = []
+        with concurrent.futures.ThreadPoolExecutor(max_workers=workers) as pool:
+            # a few experts at a time, so that at most `workers` slots beyond the kept ones are alive
+            for lo in range(0, len(todo), workers):
+                drawn = list(pool.map(lambda e: draw_slot(e, d, h, len(inner)), todo[lo:lo + workers]))
+                for e, slot in zip(todo[lo:lo + workers], drawn):
+                    if replicate:
+                        for ee in range(E):
+                            hand_over(ee, slot)
+                    else:
+                        hand_over(e, slot)
+                    if keep_host:
+                        kept.append(slot)
+        slots = kept * E if (replicate and keep_host) else kept
+    else:
+        for e in range(E):
+            hand_over(e, slots[e])
     bias = None
+    cent = torch.from_numpy(cent_host).cuda()
+    gamma = torch.from_numpy(gamma_host).cuda()
     if cfg["zipf"]:
-        bias = zipf_score_bias(x.cpu().numpy(), cent.cpu().numpy(), s=1.2)
+        bias = zipf_score_bias(x.cpu().numpy(), cent_host, s=1.2)
         plugin.set_score_bias(bias)
     plugin.configure([B, S, d])
     plugin.initialize()
     return plugin, x.view(B, S, d), cent, gamma, slots, bias
+
+
+def uniform_batch(torch, cent, rows_per_expert, like_std=1.0, key=7):
+    """A batch that the gating routes to exactly `rows_per_expert` tokens per expert (token t leans towards the
+    centroid of expert t mod E), with the scale of the ordinary batch.  The caller checks the realised counts."""
+    E, d = cent.shape
+    T = E * rows_per_expert
+    noise = torch.from_numpy(_normal((key,), (T, d))).cuda()
+    xu = 50.0 * cent[torch.arange(T, device="cuda") % E] + 0.5 * noise
+    return (xu * (like_std / xu.std())).contiguous()
 
 
 def cpu_baseline(cfg, x, cent, gamma, slots, bias, sample_tokens):
@@ -138,9 +220,29 @@ def cpu_baseline(cfg, x, cent, gamma, slots, bias, sample_tokens):
                       f"oracle/moe_cpu.c (FP32, OpenMP, AVX2), {dt:.2f} s"}
 
 
+def time_steps(torch, step, steps, warmup):
+    """W untimed steps, then K timed ones with an event between every two of them (on torch's current stream,
+    which is the stream `step` queues on).  Returns (per-step ms [K], ms from first to last event / K, host ms / K)."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t_wall = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t_wall) * 1e3 / steps
+    per_step = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
+    return per_step, marks[0].elapsed_time(marks[steps]) / steps, wall_ms
+
+
 def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None):
-    """W untimed steps, then K timed ones between two events on the layer's stream, with the library's phase
-    marks (HIP events on the same stream) kept for exactly those K steps."""
+    """Two passes of W untimed + K timed steps.  The first runs with the library's phase marks off and gives the
+    per-step times (`value` comes from their median); the second, of the same length, runs with the marks on (HIP
+    events on the layer's stream at the phase boundaries, kept for exactly its K steps) and gives the phase times
+    the roofline figures are computed from."""
     n_mat = 3 if gated else 2  # weight matrices of an expert
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = x.shape[0], x.shape[1]
@@ -160,21 +262,13 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
         def step():
             plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
 
-    plugin.set_timing(steps)  # HIP events at the phase boundaries, kept for every step of the timed region
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t_wall = time.perf_counter()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        step()
-    end.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t_wall) * 1e3 / steps
-    ms_per_step = start.elapsed_time(end) / steps
-    # per-phase averages over exactly the steps of the timed region (events recorded on the layer's stream)
+    plugin.set_timing(0)
+    per_step, mean_ms, wall_ms = time_steps(torch, step, steps, warmup)
+    plugin.set_timing(steps)
+    marked_steps, marked_mean_ms, _ = time_steps(torch, step, steps, warmup)
+    # per-phase averages over exactly the steps of the second pass
     phase_runs = plugin.timing_history(steps)
+    plugin.set_timing(0)
     assert len(phase_runs) == steps
     last = phase_runs[-1]
     phases = {k: float(np.mean([p[k] for p in phase_runs])) for k in phase_runs[0]}
@@ -189,6 +283,7 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
     launches = ("two launches per step: wi_0 and wi_1 with gelu*mul, wo with residual; figures per weight matrix"
                 if gated else "two launches per step: wi with ReLU, wo with residual")
     copies = plugin.last_streaming()[0] if not resident else 0
+    provenance = None
     if not resident and copies > 0:
         # streamed experts: the host link bounds the call, not HBM and not the matrix core (experts still in a
         # slot from the call before are not copied again)
@@ -200,21 +295,21 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
                             "bytes / expert-loop time"}
     elif few_rows:
         bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
+        traffic, provenance = (None, None) if gated else traffic_of(name, bytes_per_launch)
         roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "traffic": None if gated or name not in MEASURED_TRAFFIC_RATIO
-                    else round(MEASURED_TRAFFIC_RATIO[name] * bytes_per_launch),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": traffic,
                     "kernel": f"expert_skinny_kernel ({launches})",
                     "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     else:
         flops_per_launch = 2.0 * T * d * h
+        traffic, provenance = (None, None) if gated else traffic_of(name, 4.0 * (E * d * h + T * d + T * h))
         roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
-                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "traffic": None if gated or name not in MEASURED_TRAFFIC_RATIO
-                    else round(MEASURED_TRAFFIC_RATIO[name] * 4.0 * (E * d * h + T * d + T * h)),
+                    "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": traffic,
                     "kernel": f"expert_gemm_grouped_kernel ({launches})",
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    if provenance:
+        roofline["traffic_provenance"] = provenance
 
     # (with the rms norm of every workload here the expert norm is no phase of its own: it rides on the first
     # expert product)
@@ -230,18 +325,68 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
     phase_rates = {k: {"bytes": v, "GB/s": round(v / (phases[k] * 1e-3) / 1e9, 1),
                        "frac_of_hbm_peak": round(v / (phases[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
                    for k, v in phase_bytes.items() if phases.get(k, 0) > 0}
-    return dict(ms_per_step=ms_per_step, wall_ms=wall_ms, phases=phases, last=last, count=count, stats=stats,
-                active=active, resident=resident, roofline=roofline, phase_rates=phase_rates, tokens=T)
+    return dict(ms_per_step=float(np.median(per_step)), mean_ms=mean_ms, min_ms=float(np.min(per_step)),
+                marked_ms=float(np.median(marked_steps)), wall_ms=wall_ms, phases=phases, last=last, count=count,
+                stats=stats, active=active, resident=resident, roofline=roofline, phase_rates=phase_rates, tokens=T)
 
 
 def secondary_line(m, cfg, name):
     """What the headline line says of the primary workload, shortened, for a further workload of the same run."""
     return {"workload": f"{name}: {cfg['variant']} E={cfg['E']} d={cfg['d']} h={cfg['h']} tokens={m['tokens']}",
             "value": round(m["tokens"] / (m["ms_per_step"] * 1e-3), 1), "unit": "tokens/s",
-            "ms_per_step": round(m["ms_per_step"], 4), "active_experts": m["active"],
+            "ms_per_step": round(m["ms_per_step"], 4), "ms_per_step_with_phase_marks": round(m["marked_ms"], 4),
+            "active_experts": m["active"],
             "tokens_per_expert_min_max": [int(m["count"].min()), int(m["count"].max())],
             "roofline": m["roofline"], "phases_ms": {k: round(v, 4) for k, v in m["phases"].items()},
             "phase_rates": m["phase_rates"]}
+
+
+def sweep_point(mm, n, d, h, n_mat):
+    """One point of a sweep over rows per expert: the expert launches against both of their rooflines.  `attainable_ms`
+    is what a launch cannot beat: the active experts' weight bytes at the HBM peak or its flops at the matrix peak,
+    whichever takes longer."""
+    g_ms = (mm["phases"]["expert_gemm1"] + mm["phases"]["expert_gemm2"]) / n_mat
+    weight_bytes = mm["active"] * 4.0 * d * h
+    flops = 2.0 * n * d * h
+    attainable_ms = max(weight_bytes / (HBM_PEAK_GBS * 1e9), flops / (MFMA_FP32_PEAK_TFLOPS * 1e12)) * 1e3
+    return {"ms_per_step": round(mm["ms_per_step"], 4), "tokens_per_s": round(n / (mm["ms_per_step"] * 1e-3), 1),
+            "active_experts": mm["active"], "rows_per_expert_min_max": [int(mm["count"].min()), int(mm["count"].max())],
+            "expert_launch_ms": round(g_ms, 4), "attainable_launch_ms": round(attainable_ms, 4),
+            "frac_of_attainable": round(attainable_ms / g_ms, 4),
+            "weight_GBs": round(weight_bytes / (g_ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(weight_bytes / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "TFLOPs": round(flops / (g_ms * 1e-3) / 1e12, 2),
+            "frac_of_mfma_peak": round(flops / (g_ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4)}
+
+
+def vendor_bmm(torch, E, rows, d, h, steps, warmup):
+    """The vendor library's batched FP32 GEMM (torch.bmm) on the uniform version of the expert problem: E x
+    [rows x d] . [h x d]^T and E x [rows x h] . [d x h]^T with Gaussian operands, weights K-contiguous as the
+    layer stores them.  A comparator on the same box in the same run, not part of the product."""
+    torch.backends.cuda.matmul.allow_tf32 = False
+    out = {}
+    for label, (N, K) in (("wi", (h, d)), ("wo", (d, h))):
+        a = torch.from_numpy(_normal((50, N), (E, rows, K))).cuda()
+        b = torch.from_numpy(_normal((51, N), (E, N, K), K ** -0.5)).cuda()
+        bt = b.transpose(1, 2)
+        c = torch.empty(E, rows, N, device="cuda")
+        per_step, mean_ms, _ = time_steps(torch, lambda: torch.bmm(a, bt, out=c), steps, warmup)
+        ms = float(np.median(per_step))
+        out[label] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * E * rows * N * K / (ms * 1e-3) / 1e12, 2)}
+        del a, b, bt, c
+    total_ms = out["wi"]["ms"] + out["wo"]["ms"]
+    out["both"] = {"ms": round(total_ms, 4), "TFLOPs": round(4.0 * E * rows * d * h / (total_ms * 1e-3) / 1e12, 2)}
+    out["what"] = f"torch.bmm fp32, {E} x [{rows} x K] . [N x K]^T for (N, K) = ({h}, {d}) and ({d}, {h}), Gaussian operands"
+    return out
+
+
+def h2d_rate(torch, nbytes, reps=5):
+    """Bare rate of asynchronous host-to-device copies of `nbytes` from page-locked memory (GB/s)."""
+    src = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    src.fill_(1)
+    dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    per_step, _, _ = time_steps(torch, lambda: dst.copy_(src, non_blocking=True), reps, 2)
+    return nbytes / (float(np.median(per_step)) * 1e-3) / 1e9
 
 
 def main():
@@ -255,12 +400,14 @@ def main():
     ap.add_argument("--ffn", default="relu", choices=["relu", "gated_gelu"],
                     help="relu: the two-matrix form the headline metric is quoted on; gated_gelu: the three-matrix "
                          "form (an extra measurement, without the CPU leg)")
-    ap.add_argument("--sweep-tokens", default="",
+    ap.add_argument("--sweep-tokens", default=None,
                     help="comma-separated token counts: after the workload proper, the same layer is timed on that many "
-                         "tokens of the batch each (e.g. 256,512,1024,2048 with c2: 8 to 64 rows per expert)")
+                         "tokens of the batch each (default with c2: 256,512,1024,2048, i.e. 8 to 64 rows per expert; "
+                         "'' for none)")
     ap.add_argument("--mc", type=int, default=0, help="override the workload's max_concurrency")
     ap.add_argument("--no-secondary", action="store_true",
-                    help="with the default workload: do not also measure the decode shape (c5) and the skewed one (c4)")
+                    help="with the default workload: only the headline workload (no decode shape, streamed configuration, "
+                         "skewed workload, sweeps or vendor comparator)")
     ap.add_argument("--replicate-weights", action="store_true",
                     help="profiling aid: give every expert the values of expert 0 (short set-up, same work)")
     args = ap.parse_args()
@@ -284,9 +431,13 @@ def main():
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = cfg["shape"]
     T = B * S
+    extras = args.config == "c2" and not args.no_secondary and not gated
+    if args.sweep_tokens is None:
+        args.sweep_tokens = "256,512,1024,2048" if extras else ""
     torch.cuda.set_device(0)
-    plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=not args.no_cpu,
-                                                      replicate=args.replicate_weights)
+    # the host copies of the experts are kept for the CPU leg and for the streamed layer over the same weights
+    keep_host = (not args.no_cpu) or (extras and not args.replicate_weights)
+    plugin, x, cent, gamma, slots, bias = build_layer(torch, cfg, keep_host=keep_host, replicate=args.replicate_weights)
     stack = None
     if cfg.get("layers", 1) > 1:  # clones share the sub-layer and so the host copy of the weights
         stack = [plugin]
@@ -297,12 +448,12 @@ def main():
             stack.append(twin)
     m = measure(torch, plugin, cfg, args.config, x, args.steps, args.warmup, gated, stack=stack)
     count, stats, active, resident = m["count"], m["stats"], m["active"], m["resident"]
-    ms_per_step, wall_ms, phases, last = m["ms_per_step"], m["wall_ms"], m["phases"], m["last"]
+    ms_per_step, phases, last = m["ms_per_step"], m["phases"], m["last"]
     roofline, phase_rates = m["roofline"], m["phase_rates"]
 
     out = {
         "metric": f"MoE-layer tokens/s (E={E},d={d},h={h},fp32)",
-        "value": round(T / (ms_per_step * 1e-3), 1),
+        "value": round(T / (ms_per_step * 1e-3), 1),  # tokens through the layer (the whole stack, if stacked) per second
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -312,61 +463,132 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic" + (" (expert 0 replicated)" if args.replicate_weights else ""),
+        "data": "synthetic: numpy default_rng on SeedSequence(0) children, one per tensor, uploaded once"
+                + (" (expert 0's weights replicated to every expert)" if args.replicate_weights else ""),
         "config": {"workload": f"{args.config}: {cfg['variant']} E={E} d={d} h={h} tokens={T} ({B}x{S}) "
                                f"max_concurrency={cfg['mc']} ({'resident' if resident else 'streamed'} experts), "
                                f"T5_FF rms norm + {'gated gelu (three matrices)' if gated else 'relu'}", "tokens": T, "active_experts": active,
                    "tokens_per_expert_min_max": [int(count.min()), int(count.max())]},
+        "timing": {"value_from": "median of the per-step times of a pass with the library's phase marks off",
+                   "ms_per_step_mean": round(m["mean_ms"], 4), "ms_per_step_min": round(m["min_ms"], 4),
+                   "ms_per_step_with_phase_marks": round(m["marked_ms"], 4),
+                   "phases_from": "a second pass of the same length with the phase marks on"},
         "roofline": roofline,
         "phases_ms": {k: round(v, 4) for k, v in phases.items()},
         "phases_ms_last_timed_step": {k: round(v, 4) for k, v in last.items()},
         "phase_rates": phase_rates,
-        "host_ms_per_step": round(wall_ms, 4),
+        "host_ms_per_step": round(m["wall_ms"], 4),
         "routing": stats,
     }
     if stack:
         out["config"]["stacked_layers"] = len(stack)
-        out["value"] = round(T / (ms_per_step * 1e-3), 1)  # tokens through the whole stack per second
     if not resident:
         copies, hits = plugin.last_streaming()
         out["streaming_last_call"] = {"experts_copied": copies, "experts_found_in_slots": hits}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, x, cent, gamma, slots, bias, min(args.cpu_sample, T))
-    # Further workloads of the same run (the headline `value` above is untouched by them):
-    #   c5, the decode shape: same layer (E, d, h as c2), 64 tokens of the same batch
-    #   c4, the skewed base_layer workload: a layer of its own, built after the first is released
+
+    # Further workloads of the same run (the headline `value` above is untouched by them).
     secondary = {}
-    if args.config == "c2" and not args.no_secondary and not gated:
-        c5 = dict(CONFIGS["c5"], ffn=args.ffn)
-        x5 = x.reshape(T, d)[:64].reshape(64, 1, d).contiguous()
-        secondary["c5"] = secondary_line(measure(torch, plugin, c5, "c5", x5, max(args.steps, 50), args.warmup), c5, "c5")
-    # Few to many rows per expert on the same layer: the expert kernels' achieved weight-byte rate (they are
-    # bound by streaming the weights until an expert has some tens of rows) next to their flop rate
+
+    def extra(key, fn):  # the headline line must not depend on the extras
+        try:
+            secondary[key] = fn()
+        except Exception as exc:
+            secondary[key] = {"error": repr(exc)}
+
+    if extras:
+        # c5, the decode shape: same layer (E, d, h as c2), 64 tokens of the same batch
+        def leg_c5():
+            c5 = dict(CONFIGS["c5"], ffn=args.ffn)
+            x5 = x.reshape(T, d)[:64].reshape(64, 1, d).contiguous()
+            return secondary_line(measure(torch, plugin, c5, "c5", x5, max(args.steps, 50), args.warmup), c5, "c5")
+        extra("c5", leg_c5)
+
+        # the same layer on a batch routed to exactly T/E rows per expert, and the vendor's batched GEMM on that
+        # uniform problem: what separates the expert kernel from the best known code for the shape
+        def leg_uniform():
+            xu = uniform_batch(torch, cent, T // E, like_std=float(x.std())).view(B, S, d)
+            mu = measure(torch, plugin, cfg, None, xu, args.steps, args.warmup)
+            g1, g2 = mu["phases"]["expert_gemm1"], mu["phases"]["expert_gemm2"]
+            fl = 2.0 * T * d * h
+            return {"rows_per_expert_min_max": [int(mu["count"].min()), int(mu["count"].max())],
+                    "ms_per_step": round(mu["ms_per_step"], 4),
+                    "wi": {"ms": round(g1, 4), "TFLOPs": round(fl / (g1 * 1e-3) / 1e12, 2)},
+                    "wo": {"ms": round(g2, 4), "TFLOPs": round(fl / (g2 * 1e-3) / 1e12, 2)},
+                    "both": {"ms": round(g1 + g2, 4), "TFLOPs": round(2 * fl / ((g1 + g2) * 1e-3) / 1e12, 2)},
+                    "what": "the library's two expert launches (norm + ReLU, residual epilogues included) on a batch the "
+                            "gating routes uniformly"}
+        extra("c2_uniform", leg_uniform)
+        extra("vendor_bmm", lambda: vendor_bmm(torch, E, T // E, d, h, args.steps, args.warmup))
+
+    # Few to many rows per expert on the same layer: the expert launches against what neither roofline lets
+    # them beat (they are bound by streaming the weights until an expert has some tens of rows)
     if args.sweep_tokens:
-        sweep = {}
-        for n in [int(v) for v in args.sweep_tokens.split(",") if v]:
-            xn = x.reshape(T, d)[:n].reshape(n, 1, d).contiguous()
-            mm = measure(torch, plugin, cfg, None, xn, args.steps, args.warmup, gated)
-            g_ms = (mm["phases"]["expert_gemm1"] + mm["phases"]["expert_gemm2"]) / n_mat
-            sweep[str(n)] = {"ms_per_step": round(mm["ms_per_step"], 4), "tokens_per_s": round(n / (mm["ms_per_step"] * 1e-3), 1),
-                             "active_experts": mm["active"], "rows_per_expert_min_max": [int(mm["count"].min()), int(mm["count"].max())],
-                             "expert_launch_ms": round(g_ms, 4),
-                             "weight_GBs": round(mm["active"] * 4.0 * d * h / (g_ms * 1e-3) / 1e9, 1),
-                             "frac_of_hbm_peak": round(mm["active"] * 4.0 * d * h / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                             "TFLOPs": round(2.0 * n * d * h / (g_ms * 1e-3) / 1e12, 2),
-                             "phases_ms": {k: round(v, 4) for k, v in mm["phases"].items()}}
-        out["sweep_tokens"] = sweep
+        def leg_sweep():
+            sweep = {}
+            for n in [int(v) for v in args.sweep_tokens.split(",") if v]:
+                xn = x.reshape(T, d)[:n].reshape(n, 1, d).contiguous()
+                sweep[str(n)] = sweep_point(measure(torch, plugin, cfg, None, xn, args.steps, args.warmup, gated), n, d, h, n_mat)
+            return sweep
+        extra("sweep", leg_sweep)
+
+    if extras:
+        # c3: the same weights streamed through two slots (a second layer over the same host arrays), with the
+        # overlap efficiency max(t_copy, t_compute) / t_total: t_compute is the resident layer's expert time of
+        # this run, t_copy the streamed bytes at the bare rate of asynchronous copies of one slot
+        def leg_c3():
+            c3 = dict(CONFIGS["c3"], ffn=args.ffn)
+            p3, x3, *_ = build_layer(torch, c3, keep_host=True, slots=slots)
+            try:
+                steps3 = min(args.steps, 10)
+                m3 = measure(torch, p3, c3, "c3", x3, steps3, 2)
+                copies, hits = p3.last_streaming()
+                slot_bytes = 4 * (d + n_mat * d * h)
+                bare = h2d_rate(torch, slot_bytes)
+                t_copy = copies * slot_bytes / (bare * 1e9) * 1e3
+                t_compute = phases["expert_gemm1"] + phases["expert_gemm2"]
+                t_total = m3["ms_per_step"]
+                line = secondary_line(m3, c3, "c3")
+                line.update({"steps": steps3, "copies": copies, "hits": hits,
+                             "h2d_GBs": round(copies * slot_bytes / (t_total * 1e-3) / 1e9, 2),
+                             "bare_h2d_GBs_one_slot": round(bare, 2), "t_copy_ms": round(t_copy, 3),
+                             "t_compute_ms": round(t_compute, 3), "t_total_ms": round(t_total, 3),
+                             "overlap_efficiency": round(max(t_copy, t_compute) / t_total, 4)})
+                return line
+            finally:
+                p3.terminate()
+                p3.destroy()
+        extra("c3", leg_c3)
+
     plugin.terminate()
     plugin.destroy()
     del slots
-    if args.config == "c2" and not args.no_secondary and not gated:
-        try:
+    if extras:
+        # c4, the skewed base_layer workload: a layer of its own, built after the first is released; then the
+        # same layer without the score bias on uniformly routed batches: the expert kernels' rate against rows
+        # per expert (what an expert of each size of the skewed histogram gets)
+        def leg_c4():
             c4 = dict(CONFIGS["c4"], ffn=args.ffn)
-            p4, x4, *_ = build_layer(torch, c4, keep_host=False)
-            secondary["c4"] = secondary_line(measure(torch, p4, c4, "c4", x4.contiguous(), args.steps, args.warmup), c4, "c4")
-            p4.terminate()
-        except Exception as exc:  # the headline line must not depend on the extras
-            secondary["c4"] = {"error": repr(exc)}
+            p4, x4, cent4, *_ = build_layer(torch, c4, keep_host=False)
+            try:
+                m4 = measure(torch, p4, c4, "c4", x4.contiguous(), args.steps, args.warmup)
+                line = secondary_line(m4, c4, "c4")
+                line["tokens_per_expert"] = [int(v) for v in m4["count"]]
+                p4.set_score_bias(None)
+                table = {}
+                for rows in (16, 32, 64, 128, 256, 512, 1024, 2048):
+                    n = rows * c4["E"]
+                    xu = uniform_batch(torch, cent4, rows, like_std=float(x4.std())).view(n, 1, c4["d"])
+                    mu = measure(torch, p4, c4, None, xu, max(5, args.steps // 2), 2)
+                    pt = sweep_point(mu, n, c4["d"], c4["h"], 2)
+                    table[str(rows)] = {k: pt[k] for k in ("rows_per_expert_min_max", "expert_launch_ms", "TFLOPs",
+                                                           "frac_of_mfma_peak", "frac_of_attainable")}
+                line["expert_rate_vs_rows_per_expert"] = table
+                return line
+            finally:
+                p4.terminate()
+        extra("c4", leg_c4)
     if secondary:
         out["secondary"] = secondary
     print(json.dumps(out))
