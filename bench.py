@@ -276,7 +276,11 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
     active = int((count > 0).sum())
 
     resident = cfg["mc"] >= E
-    few_rows = T <= 16 * E  # same rule the sub-layer uses to pick the few-row kernels
+    # which roofline bounds the expert launches: streaming the active experts' weights at the HBM peak, or the
+    # flops at the matrix peak, whichever takes longer; the kernel is named by the sub-layer's own rules
+    hbm_bound = active * 4.0 * d * h / (HBM_PEAK_GBS * 1e9) > 2.0 * T * d * h / (MFMA_FP32_PEAK_TFLOPS * 1e12)
+    tile_kernel = "expert_gemm_grouped_small_kernel" if (T <= 64 * E and not gated) else "expert_gemm_grouped_kernel"
+    kernel_name = "expert_skinny_kernel" if T <= 2 * E else tile_kernel
     # average launch of the two expert kernels; the gated form's first launch takes two matrices, so its
     # figures are per matrix: (time of both launches) / 3
     gemm_ms = (phases["expert_gemm1"] + phases["expert_gemm2"]) / n_mat
@@ -293,19 +297,19 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
                     "kernel": f"host-to-device copies of {copies} of {active} active experts overlapped with expert kernels",
                     "note": "bounded by the host link (PCIe Gen5 x16, 64 GB/s per direction): achieved = streamed weight "
                             "bytes / expert-loop time"}
-    elif few_rows:
+    elif hbm_bound:
         bytes_per_launch = active * 4.0 * d * h  # one weight matrix per launch; activations are negligible
         traffic, provenance = (None, None) if gated else traffic_of(name, bytes_per_launch)
         roofline = {"bound": "hbm", "achieved": round(bytes_per_launch / (gemm_ms * 1e-3) / 1e9, 2),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "traffic": traffic,
-                    "kernel": f"expert_skinny_kernel ({launches})",
+                    "kernel": f"{kernel_name} ({launches})",
                     "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     else:
         flops_per_launch = 2.0 * T * d * h
         traffic, provenance = (None, None) if gated else traffic_of(name, 4.0 * (E * d * h + T * d + T * h))
         roofline = {"bound": "mfma", "achieved": round(flops_per_launch / (gemm_ms * 1e-3) / 1e12, 3),
                     "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "traffic": traffic,
-                    "kernel": f"expert_gemm_grouped_kernel ({launches})",
+                    "kernel": f"{kernel_name} ({launches})",
                     "algorithmic_flops_per_launch": flops_per_launch, "avg_launch_ms": round(gemm_ms, 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     if provenance:
@@ -405,6 +409,9 @@ def main():
                          "tokens of the batch each (default with c2: 256,512,1024,2048, i.e. 8 to 64 rows per expert; "
                          "'' for none)")
     ap.add_argument("--mc", type=int, default=0, help="override the workload's max_concurrency")
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="run the workload on the first N tokens of its batch only (as one sequence per token), e.g. to "
+                         "profile a point of the token sweep by itself")
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: only the headline workload (no decode shape, streamed configuration, "
                          "skewed workload, sweeps or vendor comparator)")
@@ -446,7 +453,11 @@ def main():
             twin.configure([B, S, d])
             twin.initialize()
             stack.append(twin)
-    m = measure(torch, plugin, cfg, args.config, x, args.steps, args.warmup, gated, stack=stack)
+    if 0 < args.tokens < T:
+        x = x.reshape(T, d)[:args.tokens].reshape(args.tokens, 1, d).contiguous()
+        B, S, T = args.tokens, 1, args.tokens
+        extras = False
+    m = measure(torch, plugin, cfg, args.config if not args.tokens else None, x, args.steps, args.warmup, gated, stack=stack)
     count, stats, active, resident = m["count"], m["stats"], m["active"], m["resident"]
     ms_per_step, phases, last = m["ms_per_step"], m["phases"], m["last"]
     roofline, phase_rates = m["roofline"], m["phase_rates"]

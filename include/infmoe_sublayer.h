@@ -157,6 +157,10 @@ class MoESubLayer {
     virtual Status runGrouped(const GroupedRun& g);
     /* Whether runGrouped honours g.weights / g.expertSlot (the default one does). */
     virtual bool groupedFromSlots() const { return true; }
+    /* rowTileHeight() for a call of `tokenCount` tokens, for a sub-layer that cuts the rows of calls with few rows
+     * per expert into shorter tiles (a multiple of 16, at most rowTileHeight(), at least minRowTileHeight()). */
+    virtual int rowTileHeightFor(int32_t /*tokenCount*/) const { return rowTileHeight(); }
+    virtual int minRowTileHeight() const { return rowTileHeight(); }
     int expertCount() const { return mExpertCount; }
 
    private:

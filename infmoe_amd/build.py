@@ -27,6 +27,10 @@ SOURCES = [
     "kernels/expert_gemm_one_relu.hip",
     "kernels/expert_gemm_grouped.hip",
     "kernels/expert_gemm_one.hip",
+    "kernels/expert_gemm_small_grouped_relu.hip",
+    "kernels/expert_gemm_small_grouped.hip",
+    "kernels/expert_gemm_small_one_relu.hip",
+    "kernels/expert_gemm_small_one.hip",
     "kernels/expert_gemm.hip",
     "kernels/gating.hip",
     "kernels/gating_slab.hip",

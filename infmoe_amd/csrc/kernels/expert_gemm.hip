@@ -62,10 +62,15 @@ bool fast_path_ok(const GemmProblem& p) {
     return p.K % 32 == 0 && (bits & 15) == 0 && (reinterpret_cast<uintptr_t>(p.row_stats) & 7) == 0;
 }
 
-// the second product needs its residual, the two-matrix form its second matrix
+// the second product needs its residual, the two-matrix form its second matrix (and its tall tiles)
 bool operands_ok(const GemmProblem& p) {
     if (p.epilogue == EPI_RESIDUAL) return p.R != nullptr;
-    return p.epilogue != EPI_GATED_GELU || p.B1 != nullptr;
+    return p.epilogue != EPI_GATED_GELU || (p.B1 != nullptr && !p.small_tiles);
+}
+
+// LDS of the few-rows-per-expert form: 32-float steps (rows of 36 floats), one weight matrix
+size_t lds_bytes_small(int a_alloc_rows) {
+    return 2 * ((size_t)a_alloc_rows + kGemmColumns) * 36 * sizeof(float);
 }
 
 }  // namespace
@@ -85,7 +90,8 @@ hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t wei
 
 hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
-    if (tile_rows <= 0 || tile_rows % 16 != 0 || tile_rows > gemm_tile_rows(p.epilogue)) return hipErrorInvalidValue;
+    if (tile_rows <= 0 || tile_rows % 16 != 0 || tile_rows > gemm_tile_rows(p.epilogue, p.small_tiles != 0))
+        return hipErrorInvalidValue;
     if (!operands_ok(p)) return hipErrorInvalidValue;
     if (!fast_path_ok(p)) {
         const size_t n = (size_t)rows * p.N;
@@ -95,6 +101,13 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hip
     const int tile = std::min(row_tile_height(rows, tile_rows), ((rows + 15) / 16) * 16);
     const int a_alloc = ((tile + 31) / 32) * 32;  // whole 32-row slabs
     const dim3 grid((p.N + kGemmColumns - 1) / kGemmColumns, (rows + tile - 1) / tile);
+    if (p.small_tiles) {
+        // (LDS for the tallest tile of this form whatever this expert's height: the two-workgroups-per-unit
+        // residency is the same for every launch of the form)
+        const size_t lds = lds_bytes_small(kGemmTileRowsSmall);
+        return p.epilogue == EPI_RELU ? expert_gemm_launch_small_one_relu(p, rows, tile, kGemmTileRowsSmall, grid, lds, stream)
+                                      : expert_gemm_launch_small_one(p, rows, tile, kGemmTileRowsSmall, grid, lds, stream);
+    }
     const bool gated = p.epilogue == EPI_GATED_GELU;
     const size_t lds = lds_bytes(gated, a_alloc, p.K);
     return gated ? expert_gemm_launch_one_gated(p, rows, tile, a_alloc, grid, lds, stream)
@@ -108,6 +121,12 @@ hipError_t launch_expert_gemm_grouped(const GemmProblem& p, size_t weight_stride
     if (!expert_gemm_grouped_ok(p, weight_stride) || !operands_ok(p)) return hipErrorInvalidValue;  // see launch_expert_gemm_any_shape_grouped
     const int n_col_tiles = (p.N + kGemmColumns - 1) / kGemmColumns;
     const dim3 grid((unsigned)kXcdCount * (unsigned)xcd_tile_capacity(max_tiles) * (unsigned)n_col_tiles);
+    if (p.small_tiles) {
+        const size_t lds = lds_bytes_small(kGemmTileRowsSmall);
+        return p.epilogue == EPI_RELU
+                   ? expert_gemm_launch_small_grouped_relu(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream)
+                   : expert_gemm_launch_small_grouped(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream);
+    }
     const bool gated = p.epilogue == EPI_GATED_GELU;
     const size_t lds = lds_bytes(gated, gated ? kGemmTileRowsGated : kGemmTileRows, p.K);
     return gated ? expert_gemm_launch_grouped_gated(p, weight_stride, tiles, sched, n_col_tiles, grid, lds, stream)

@@ -23,6 +23,17 @@ hipError_t expert_gemm_launch_grouped(const GemmProblem& p, size_t weight_stride
 hipError_t expert_gemm_launch_grouped_relu(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
                                            const int* sched, int n_col_tiles, dim3 grid, size_t lds,
                                            hipStream_t stream);
+// the few-rows-per-expert form (two workgroups per compute unit)
+hipError_t expert_gemm_launch_small_one(const GemmProblem& p, int rows, int tile_rows, int a_alloc_rows, dim3 grid,
+                                        size_t lds, hipStream_t stream);
+hipError_t expert_gemm_launch_small_one_relu(const GemmProblem& p, int rows, int tile_rows, int a_alloc_rows, dim3 grid,
+                                             size_t lds, hipStream_t stream);
+hipError_t expert_gemm_launch_small_grouped(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
+                                            const int* sched, int n_col_tiles, dim3 grid, size_t lds,
+                                            hipStream_t stream);
+hipError_t expert_gemm_launch_small_grouped_relu(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
+                                                 const int* sched, int n_col_tiles, dim3 grid, size_t lds,
+                                                 hipStream_t stream);
 hipError_t expert_gemm_launch_grouped_gated(const GemmProblem& p, size_t weight_stride, const RowTile* tiles,
                                             const int* sched, int n_col_tiles, dim3 grid, size_t lds,
                                             hipStream_t stream);

@@ -506,5 +506,69 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProbl
                            GATED ? kGemmTileRowsGated : kGemmTileRows);
 }
 
+// ---- Calls with few rows per expert (gemm_small_tiles(): tokens <= 64 * experts).
+// The kernels above keep one workgroup per compute unit: their registers and LDS are sized for tiles of 256
+// rows.  A tile of a few dozen rows has little arithmetic per byte of weights; what it needs is bytes in
+// flight and no dead time, and a workgroup by itself has dead time: its start (nothing computes until the
+// first loads are back), its end (nothing loads while the last tile is stored) and the turn of every barrier.
+// Here the same tile body is instantiated for tiles of up to kGemmTileRowsSmall rows only - 32-float steps,
+// few accumulators, half the LDS - so that TWO workgroups share a compute unit and each fills the other's gaps
+// (the second launch bound below asks the compiler to stay within the registers of two waves per SIMD).
+// Row counts are padded to 4 (whole 16-row units plus one or two 4-row groups) from 32 rows on, to 16 below.
+// Which path a call takes depends on (tokens, experts) only, so every schedule of a layer agrees on it.
+template <int BN, int EPI>
+__device__ __forceinline__ void gemm_dispatch_small(const float* A, const float* R, float* C, int rows, const float* B0,
+                                                    int n0, int N, int K, const float* stats, float* smem,
+                                                    int a_alloc_rows) {
+    static_assert(EPI != EPI_GATED_GELU, "the two-matrix form keeps its tall tiles");
+    constexpr int kMaxMb = kGemmTileRowsSmall / 16;
+    const int full = rows >> 4, rem = rows & 15;
+    int nmb = (rows + 15) >> 4, g4 = 0;
+    if (rem != 0 && rem <= 8 && full >= 2) nmb = full, g4 = (rem + 3) >> 2;
+#define INFMOE_SMALL_G(n, g)                                                                                          \
+    case 4 * (n) + (g):                                                                                               \
+        if constexpr ((n) <= kMaxMb && ((g) == 0 || ((n) >= 2 && (n) < kMaxMb)))                                      \
+            gemm_tile<n, g, BN, EPI, 32, depth_of(n, g)>(A, R, C, rows, B0, nullptr, n0, N, K, stats, smem,           \
+                                                         a_alloc_rows);                                              \
+        break;
+#define INFMOE_SMALL(n) INFMOE_SMALL_G(n, 0) INFMOE_SMALL_G(n, 1) INFMOE_SMALL_G(n, 2)
+    switch (4 * nmb + g4) {
+        INFMOE_SMALL(1) INFMOE_SMALL(2) INFMOE_SMALL(3) INFMOE_SMALL(4) INFMOE_SMALL(5) INFMOE_SMALL(6)
+        default: break;
+    }
+#undef INFMOE_SMALL
+#undef INFMOE_SMALL_G
+}
+
+template <int BN, int EPI>
+__global__ __launch_bounds__(kThreads, 2) void expert_gemm_small_kernel(GemmProblem p, int rows_total, int tile_rows,
+                                                                        int a_alloc_rows) {
+    extern __shared__ __align__(16) float smem[];
+    const int row0 = blockIdx.y * tile_rows;
+    const int rows = min(tile_rows, rows_total - row0);
+    const int n0 = blockIdx.x * BN;
+    gemm_dispatch_small<BN, EPI>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
+                                 p.C + (size_t)row0 * p.N, rows, p.B, n0, p.N, p.K,
+                                 p.row_stats ? p.row_stats + 2 * (size_t)row0 : nullptr, smem, a_alloc_rows);
+}
+
+// (the same map from workgroup id to (row tile, column tile) as expert_gemm_grouped_kernel)
+template <int BN, int EPI>
+__global__ __launch_bounds__(kThreads, 2) void expert_gemm_grouped_small_kernel(GemmProblem p, size_t weight_stride,
+                                                                                const RowTile* __restrict__ tiles,
+                                                                                const int* __restrict__ sched,
+                                                                                int n_col_tiles) {
+    extern __shared__ __align__(16) float smem[];
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
+    if (slot >= share * n_col_tiles) return;
+    const RowTile rt = tiles[first + slot / n_col_tiles];
+    const int n0 = (slot % n_col_tiles) * BN;
+    const int owner = p.expert_slot ? p.expert_slot[rt.expert] : rt.expert;
+    gemm_dispatch_small<BN, EPI>(p.A + (size_t)rt.row0 * p.K, p.R ? p.R + (size_t)rt.row0 * p.N : nullptr,
+                                 p.C + (size_t)rt.row0 * p.N, rt.rows, p.B + (size_t)owner * weight_stride, n0, p.N, p.K,
+                                 p.row_stats ? p.row_stats + 2 * (size_t)rt.row0 : nullptr, smem, kGemmTileRowsSmall);
+}
+
 }  // namespace
 }  // namespace infmoe

@@ -169,6 +169,9 @@ struct GemmProblem {
     // grouped launches only: null, or [E] where expert e's weights are at B + expert_slot[e] * weight_stride
     // instead of B + e * weight_stride (experts held in slots in whatever order they arrived)
     const int* expert_slot;
+    // nonzero: the call has few rows per expert (gemm_small_tiles()) and its tiles, of at most kGemmTileRowsSmall
+    // rows, go to the kernels that run two workgroups per compute unit.  Not with EPI_GATED_GELU.
+    int small_tiles;
 };
 // One expert, `rows` known on the host, cut into row tiles of at most `tile_rows` rows (a multiple of
 // 16 no larger than gemm_tile_rows(p.epilogue); both launches of a sub-layer pass the same value so
@@ -186,7 +189,17 @@ hipError_t launch_expert_gemm_any_shape_grouped(const GemmProblem& p, size_t wei
                                                 int rows, hipStream_t stream);
 constexpr int kGemmTileRows = 256;       // tallest row tile of the GEMM kernel
 constexpr int kGemmTileRowsGated = 192;  // ... of its two-matrix (gated) form (two accumulator sets)
-inline int gemm_tile_rows(int epilogue) { return epilogue == EPI_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
+constexpr int kGemmTileRowsSmall = 96;   // ... of the form for calls with few rows per expert
+inline int gemm_tile_rows(int epilogue, bool small_tiles = false) {
+    return epilogue == EPI_GATED_GELU ? kGemmTileRowsGated : (small_tiles ? kGemmTileRowsSmall : kGemmTileRows);
+}
+// Whether a layer call of `tokens` tokens over `experts` experts takes the few-rows-per-expert form of the
+// matrix-core kernels (on average at most 64 rows per expert; an expert with more than kGemmTileRowsSmall is
+// cut into several tiles).  A function of the call's shape only: the grouped and the per-expert schedule of a
+// layer have to pick the same kernel for the same expert to agree bit for bit.
+inline bool gemm_small_tiles(int tokens, int experts, int ffn_kind) {
+    return ffn_kind != FFN_GATED_GELU && (long long)tokens <= 64ll * experts;
+}
 
 // Few-row experts (decode): every weight row is streamed once and dotted with up to
 // kSkinnyMaxRows activation rows held in LDS.

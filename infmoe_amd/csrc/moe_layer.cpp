@@ -158,7 +158,7 @@ Status MoELayer::carve(int T, void* workspace, Carve* c) const {
     c->sel = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
     c->pos = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
     c->rowExpert = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (size_t)T));
-    c->maxTiles = max_row_tiles(T, E, mSublayer->rowTileHeight());
+    c->maxTiles = max_row_tiles(T, E, mSublayer->minRowTileHeight());  // room for the shortest tiles any call may be cut into
     c->tiles = reinterpret_cast<RowTile*>(take(sizeof(RowTile) * 2 * (size_t)c->maxTiles));
     c->sched = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kSchedInts));
     c->countScratch = take(expert_count_scratch_bytes(T, E));
@@ -371,7 +371,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     const bool grouped = resident();
     const int skinnyMax = mSublayer->skinnyMaxRows(T);
     INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, c.tiles, c.sched,
-                                   mSublayer->rowTileHeight(), skinnyMax, c.rowExpert, stream));
+                                   mSublayer->rowTileHeightFor(T), skinnyMax, c.rowExpert, stream));
     INFMOE_TRY(mark(2));
     // experts see the raw input (:354); the statistics of their row norm are taken while the rows are copied
     INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream, c.rowStats, mSublayer->rowStatsKind()));
@@ -382,13 +382,14 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     GroupedRun g;
     g.tokenCount = T, g.input = c.routed, g.output = c.post, g.workspace = c.subWs;
     g.count = dCount, g.offset = dOffset, g.rowExpert = c.rowExpert, g.rowStats = c.rowStats;
-    g.tiles = c.tiles, g.sched = c.sched, g.maxTiles = c.maxTiles, g.stream = stream;
+    g.tiles = c.tiles, g.sched = c.sched, g.stream = stream;
+    g.maxTiles = std::min(c.maxTiles, max_row_tiles(T, E, mSublayer->rowTileHeightFor(T)));  // of this call's tile height
     if (skinnyMax > 0) {
         // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
         // of them, each with one tile more than its rows fill.  A decode call then launches a small
         // grid (or none) for the matrix-core kernel instead of one sized for E experts.
         const int tall = T / (skinnyMax + 1);
-        g.maxTiles = std::min(c.maxTiles, tall + T / mSublayer->rowTileHeight());
+        g.maxTiles = std::min(g.maxTiles, tall + T / mSublayer->rowTileHeightFor(T));
     }
     if (timed) g.afterNorm = marks[4], g.afterGemm1 = marks[5];
     if (grouped) {

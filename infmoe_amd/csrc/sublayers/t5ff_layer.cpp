@@ -194,7 +194,10 @@ Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
 // Few-row kernels are used for an expert only when the whole call is decode-like, and the rule
 // depends on nothing but (tokens of the call, experts, rows of the expert), so that the grouped
 // and the per-expert schedules pick the same kernel for the same expert and agree bit for bit.
-static bool decode_like(int layerTokens, int expertCount) { return layerTokens <= 16 * expertCount; }
+// (Up to two tokens per expert.  With more, the matrix-core kernel for calls with few rows per expert, which runs
+// two workgroups per compute unit, streams the weights faster than the few-row kernel and one more launch
+// would: 128 tokens over 32 experts of 4096 x 10240 take 0.80 ms per launch against 0.95 ms.)
+static bool decode_like(int layerTokens, int expertCount) { return layerTokens <= 2 * expertCount; }
 
 int T5FFLayer::skinnyMaxRows(int32_t tokenCount) const {
     return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kSkinnyMaxRows : 0;
@@ -239,8 +242,10 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
         INFMOE_HIP(launch_expert_skinny(g1, rows, stream));
         INFMOE_HIP(launch_expert_skinny(g2, rows, stream));
     } else {
-        // both launches cut the rows as the grouped schedule does (rowTileHeight())
-        const int tileRows = ffnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows;
+        // both launches cut the rows, and pick their kernel, as the grouped schedule does (rowTileHeightFor())
+        const bool smallTiles = gemm_small_tiles(layerTokens, expertCount, ffnKind);
+        g1.small_tiles = g2.small_tiles = smallTiles ? 1 : 0;
+        const int tileRows = smallTiles ? kGemmTileRowsSmall : (ffnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows);
         INFMOE_HIP(launch_expert_gemm(g1, rows, tileRows, stream));
         INFMOE_HIP(launch_expert_gemm(g2, rows, tileRows, stream));
     }
@@ -250,8 +255,9 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
 Status T5FFLayer::run(int32_t tokenCount, const void* weights, const void* input, void* output, void* workspace,
                       hipStream_t stream) {
     // outside a layer call the expert stands alone: a call of tokenCount tokens over one expert, on a slot
-    // that copyWeights filled
-    return runOne(tokenCount, tokenCount, 1, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
+    // that copyWeights filled.  With up to kSkinnyMaxRows rows it is a decode call whatever the rule for
+    // layers says of (tokens, 1 expert): one expert's column tiles would occupy a third of the compute units.
+    return runOne(tokenCount, tokenCount <= kSkinnyMaxRows ? 1 : tokenCount, 1, mEmbeddingSize, mHiddenSize, mNormKind, mFfnKind, weights,
                   static_cast<const float*>(input), static_cast<float*>(output), workspace, stream, folds(), nullptr);
 }
 
@@ -292,6 +298,7 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     g2.A = hid, g2.B = w + d + (mFfnKind == FFN_GATED_GELU ? 2 : 1) * dh, g2.R = g.input, g2.C = g.output, g2.N = d, g2.K = h;
     g2.epilogue = EPI_RESIDUAL;
     const bool skinny = skinnyMaxRows(T) > 0;
+    g1.small_tiles = g2.small_tiles = gemm_small_tiles(T, mExpertCount, mFfnKind) ? 1 : 0;
     if (g.afterNorm) INFMOE_HIP(hipEventRecord(g.afterNorm, g.stream));
     if (!expert_gemm_grouped_ok(g1, stride) || !expert_gemm_grouped_ok(g2, stride)) {
         // sizes the matrix-core kernel does not take (d or h not a multiple of 32)

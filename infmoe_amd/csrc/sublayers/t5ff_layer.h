@@ -52,6 +52,10 @@ class T5FFLayer : public MoESubLayer {
     size_t residentStride() const override { return deviceStride(); }
     int skinnyMaxRows(int32_t tokenCount) const override;
     int rowTileHeight() const override { return mFfnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRows; }
+    int rowTileHeightFor(int32_t tokenCount) const override {
+        return gemm_small_tiles(tokenCount, mExpertCount, mFfnKind) ? kGemmTileRowsSmall : rowTileHeight();
+    }
+    int minRowTileHeight() const override { return mFfnKind == FFN_GATED_GELU ? kGemmTileRowsGated : kGemmTileRowsSmall; }
     Status runGrouped(const GroupedRun& g) override;
 
     // used by the kernel-level C entry points

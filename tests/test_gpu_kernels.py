@@ -239,8 +239,10 @@ def test_t5ff_row_counts(lib, torch_cuda, rows, d, h):
 
 # the benchmark's K (4096 into the first product, 10240 into the second) at the row counts of decode batches of
 # a few hundred tokens: few-row kernel (5), one 16-row unit (12), one unit + two 4-row groups... (24 -> 2 units),
-# three units (48), a 32-row block + a 16-row block + a group (52)
-@pytest.mark.parametrize("rows", [5, 12, 24, 48, 52])
+# three units (48), a 32-row block + a 16-row block + a group (52); every row count from 9 to 64 takes the
+# few-rows-per-expert form of the matrix-core kernel (a call of at most 64 rows per expert): all of its tile
+# shapes - one to four 16-row units, and from 32 rows on whole units plus one or two 4-row groups - are met
+@pytest.mark.parametrize("rows", [5, 9, 12, 16, 17, 24, 31, 33, 36, 40, 41, 48, 52, 57, 64])
 def test_t5ff_row_counts_at_full_width(lib, torch_cuda, rows):
     d, h = 4096, 10240
     w = O.draw_expert(26, 0, d, h, "relu")

@@ -119,7 +119,7 @@ def test_variants_streamed_and_resident(torch_cuda, variant, norm, ffn, mc):
     plugin.terminate()
 
 
-@pytest.mark.parametrize("shape", [(4, 128), (1, 24)])  # matrix-core tiles; few-row kernel
+@pytest.mark.parametrize("shape", [(4, 128), (1, 24), (1, 8)])  # matrix-core tiles, tall and short; few-row kernel
 @pytest.mark.parametrize("norm", ["centered", "rms"])
 def test_rows_with_a_large_mean_and_weights_with_a_common_sign(torch_cuda, shape, norm):
     """Rows with a mean of several standard deviations against weights that all have one sign: x W'^T and
@@ -143,16 +143,24 @@ def test_rows_with_a_large_mean_and_weights_with_a_common_sign(torch_cuda, shape
     plugin.terminate()
 
 
+# 300 tokens over 5 experts: the few-rows-per-expert kernels (tokens <= 64 * experts); 320 tokens with a score
+# bias that sends most of them to expert 0: the same kernels with an expert cut into several 96-row tiles next to
+# experts of a few rows; 600 tokens: the tall-tile kernels
+@pytest.mark.parametrize("shape,skew", [((2, 150), 0.0), ((2, 160), 0.6), ((4, 150), 0.0)])
 @pytest.mark.parametrize("variant", ["cpm_2", "base_layer"])
-def test_output_is_bit_identical_for_every_max_concurrency(torch_cuda, variant):
+def test_output_is_bit_identical_for_every_max_concurrency(torch_cuda, variant, shape, skew):
     """Streamed experts run one set of launches per expert, resident ones one grouped set: same
     arithmetic, same bits."""
     torch = torch_cuda
-    shape, E, d, h = (2, 150), 5, 64, 192
+    E, d, h = 5, 64, 192
+    bias = np.array([skew, 0, 0, 0, 0], np.float32) if skew else None
     outs = []
     for mc in (1, 2, 3, 5, 9):
-        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, variant, seed=8)
-        outs.append(plugin.forward(dev(torch, x.reshape(2, 150, d))).cpu().numpy())
+        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, variant, seed=8, bias=bias)
+        if mc == 5:
+            y, ref, count, _ = run_and_check(torch, plugin, x, c, g, ws, shape, variant, bias=bias)
+            assert not skew or (count.max() > 96 and count.min() < 40), count
+        outs.append(plugin.forward(dev(torch, x.reshape(*shape, d))).cpu().numpy())
         plugin.terminate()
     for o in outs[1:]:
         np.testing.assert_array_equal(o, outs[0])
@@ -242,14 +250,22 @@ def test_output_may_alias_input(torch_cuda):
     plugin.terminate()
 
 
-def test_decode_shape_uses_few_row_kernels_and_matches(torch_cuda):
-    # 24 tokens over 8 experts: some experts get 0 rows, most 1..8, possibly one above 8
-    shape, E, d, h = (24, 1), 8, 256, 640
-    for mc in (8, 2):
-        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "cpm_2", seed=13)
-        y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "cpm_2")
-        assert count.min() >= 0 and count.sum() == 24
+@pytest.mark.parametrize("skew", [0.0, 1.5])
+def test_decode_shape_uses_few_row_kernels_and_matches(torch_cuda, skew):
+    """Up to two tokens per expert: experts of up to 8 rows go to the few-row kernel.  32 tokens over 16 experts:
+    some experts get no rows, most 1..5; with a score bias one gets more than 8 and goes to the matrix-core
+    kernel in the same call.  Both schedules, same bits."""
+    shape, E, d, h = (32, 1), 16, 256, 640
+    bias = np.array([0, 0, 0, skew] + [0] * 12, np.float32) if skew else None
+    outs = []
+    for mc in (16, 2):
+        plugin, x, c, g, ws = make_layer(shape, E, d, h, mc, "cpm_2", seed=13, bias=bias)
+        y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "cpm_2", bias=bias)
+        assert count.sum() == 32 and ((count > 0) & (count <= 8)).any()
+        assert not skew or count.max() > 8, count
+        outs.append(y)
         plugin.terminate()
+    np.testing.assert_array_equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("ffn", ["relu", "gated_gelu"])
