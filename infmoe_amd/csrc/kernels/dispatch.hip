@@ -440,7 +440,7 @@ size_t expert_count_scratch_bytes(int T, int E) {
 
 hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
                                RowTile* tiles, int* sched, int tile_rows, int skinny_max, int* row_expert,
-                               hipStream_t stream) {
+                               hipStream_t stream, bool hist_ready) {
     const int nblk = (T + kCountBlockTokens - 1) / kCountBlockTokens;
     int* blockhist = static_cast<int*>(scratch);
     const size_t lds = (size_t)E * sizeof(int);
@@ -451,7 +451,7 @@ hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* coun
                                                              skinny_max, row_expert);
         return hipGetLastError();
     }
-    if (nblk > 0) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
+    if (nblk > 0 && !hist_ready) hist_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist);
     scan_kernel<<<1, kThreads, 3 * lds, stream>>>(T, E, nblk, blockhist, count, offset, tiles, sched, max_tiles,
                                             xcd_tile_capacity(max_tiles), tile_rows, skinny_max);
     if (nblk > 0) rank_kernel<<<nblk, kThreads, lds, stream>>>(T, E, sel, blockhist, offset, pos, row_expert);

@@ -17,8 +17,10 @@
 //     block per wave, 6.6 TB/s with two).
 // The chunk length shrinks as M grows (2048, 2048, 512, 256 floats for M = 1, 2, 4, 8) so that
 // activations + loads in flight + accumulators stay within 168 registers.
-// Experts outside 1..kSkinnyMaxRows rows are skipped, so the grouped launch can run next to the
-// matrix-core launch: each expert is processed by exactly one of the two.
+// An expert with more than kSkinnyMaxRows rows is done in runs of kSkinnyMaxRows rows (the last run takes what is
+// left), each a pass over the expert's weights: in a decode call (at most two tokens per expert) such an expert is
+// rare and its rows are rows that other experts did not get, so the passes cost no more than the experts they
+// replace, and the call needs no launch of the matrix-core kernel whose grid would have to be sized for it.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -192,22 +194,24 @@ __global__ __launch_bounds__(kThreads, EPI == EPI_GATED_GELU ? 2 : 3) void exper
         B0 += (size_t)owner * weight_stride;
         if (GATED) B1 += (size_t)owner * weight_stride;
     }
-    if (rows <= 0 || rows > kSkinnyMaxRows) return;
-    const float* A = p.A + (size_t)row0 * p.K;
-    const float* R = p.R ? p.R + (size_t)row0 * p.N : nullptr;
-    float* C = p.C + (size_t)row0 * p.N;
-    const float* stats = EPI != EPI_RESIDUAL && p.row_stats != nullptr ? p.row_stats + 2 * (size_t)row0 : nullptr;
-    // One body per row count: a row more than needed would cost its loads of the activation chunk
-    // again for every block of weight rows (with 5 rows in the 8-row body, 60 % more of them).
-    switch (rows) {
-        case 1: skinny_body<1, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 2: skinny_body<2, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 3: skinny_body<3, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 4: skinny_body<4, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 5: skinny_body<5, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 6: skinny_body<6, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        case 7: skinny_body<7, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
-        default: skinny_body<8, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+#pragma unroll 1
+    for (; rows > 0; rows -= kSkinnyMaxRows, row0 += kSkinnyMaxRows) {  // (a body returns when its wave has no weight rows left)
+        const float* A = p.A + (size_t)row0 * p.K;
+        const float* R = p.R ? p.R + (size_t)row0 * p.N : nullptr;
+        float* C = p.C + (size_t)row0 * p.N;
+        const float* stats = EPI != EPI_RESIDUAL && p.row_stats != nullptr ? p.row_stats + 2 * (size_t)row0 : nullptr;
+        // One body per row count: a row more than needed would cost its loads of the activation chunk
+        // again for every block of weight rows (with 5 rows in the 8-row body, 60 % more of them).
+        switch (min(rows, kSkinnyMaxRows)) {
+            case 1: skinny_body<1, 8, 2, EPI>(A, R, C, 1, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 2: skinny_body<2, 8, 2, EPI>(A, R, C, 2, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 3: skinny_body<3, 2, 8, EPI>(A, R, C, 3, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 4: skinny_body<4, 2, 8, EPI>(A, R, C, 4, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 5: skinny_body<5, 1, 8, EPI>(A, R, C, 5, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 6: skinny_body<6, 1, 8, EPI>(A, R, C, 6, B0, B1, p.N, p.K, stats, row_blocks); break;
+            case 7: skinny_body<7, 1, 8, EPI>(A, R, C, 7, B0, B1, p.N, p.K, stats, row_blocks); break;
+            default: skinny_body<8, 1, 8, EPI>(A, R, C, 8, B0, B1, p.N, p.K, stats, row_blocks); break;
+        }
     }
 }
 
@@ -228,7 +232,7 @@ int row_blocks_for(int K) {
 
 hipError_t launch_expert_skinny(const GemmProblem& p, int rows, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
-    if (rows > kSkinnyMaxRows || !fast_path_ok(p)) return hipErrorInvalidValue;
+    if (!fast_path_ok(p)) return hipErrorInvalidValue;
     const int rb = row_blocks_for(p.K), rows_per_wg = RW * kWaves * rb;
     const dim3 grid((p.N + rows_per_wg - 1) / rows_per_wg, 1);
     if (p.epilogue == EPI_GATED_GELU)

@@ -80,6 +80,7 @@ struct GateArgs {
     int steps_per;  // K chunks per slice
     int* nan_flag;    // null, or an int (host memory the device can write) set to nan_value when a token has no orderable score
     int nan_value;
+    float err_depth;  // n of the error bound of a score (see gate_err_depth)
     float* partials;  // [slices][T][E + 2]: dot products, row sum, row sum of squares
     float* gpart;     // [groups][slices][2E]: sum and sum of squares of the folded centroid slice
     int* zero_stats;  // GATE_SLICES only: null, or the 4 ints the later combine launch counts into, set to zero here
@@ -512,7 +513,7 @@ __global__ __launch_bounds__(kThreads) void gate_top1_kernel(const GateArgs arg)
             } else {
                 sel[t] = I;
                 coeff[t] = B;
-                const float bound = 8.f * FLT_EPSILON * s_rstd[tid] * s_xnorm[tid] * s_cnmax;
+                const float bound = arg.err_depth * FLT_EPSILON * s_rstd[tid] * s_xnorm[tid] * s_cnmax;  // see gate_err_depth
                 s_thr[tid] = fmaxf(bound, 4e-6f * fabsf(B));
                 if (E > 1 && (B - S2) < s_thr[tid]) s_rescue[tid] = 1;
             }
@@ -770,6 +771,28 @@ struct GatePlan {
 
 constexpr int nblk_for(int E) { return E <= 16 ? 1 : (E <= 32 ? 2 : (E <= 64 ? 4 : 8)); }
 
+}  // namespace
+
+// Which two scores FP32 can order.  A score is rstd * (sum_k x_k (g c)_k [- mu * sum_k (g c)_k]); every path here
+// forms the sum as chains of matrix-core accumulations (one instruction adds four products to a running sum),
+// two chains per slice added once, then the slices (and, in one form, the four waves' quarters) in a fixed
+// order.  For a summation of that shape the standard bound is |computed - exact| <= n u sum_k |x_k (g c)_k|
+// with u = 2^-24 and n the longest chain of roundings a term passes through: the chain's length (slice / 8
+// instructions), three roundings inside an instruction, one for the product g c held in FP32, one for the two
+// chains, the slices, the waves.  By Cauchy-Schwarz sum_k |x_k (g c)_k| <= |x| |g c|, so each score is within
+// n u rstd |x| max_e |g c_e| of its exact value, and two scores further apart than twice that - n eps rstd |x|
+// max|g c|, eps = 2 u = FLT_EPSILON - are ordered as the exact ones.  The centered norm subtracts mu * sum (g c):
+// the error of mu, at most n u |x| / sqrt(d), times |sum g c| <= sqrt(d) |g c| has the same form once more, so n
+// doubles.  n comes from the launch plan (`err_depth`).  This is a worst-case bound: a token inside it (about
+// one in 400 for Gaussian scores at d = 4096) is re-scored in float64, which costs its workgroup one sweep over
+// the row.  (The factor was 8 before, an empirical value a tenth of the bound.)
+float gate_err_depth(int slice_floats, int slices, int norm_kind) {
+    const float n = (float)(slice_floats / 8 + slices + 3 + 1 + 1 + 3);
+    return norm_kind == NORM_CENTERED ? 2.f * n : n;
+}
+
+namespace {
+
 GatePlan gate_plan(int T, int d, int E, bool vec, size_t scratch_floats) {
     const int nblk = nblk_for(E);
     const int W = E + 2;
@@ -806,6 +829,8 @@ template <int NBLK>
 hipError_t launch_nblk(GateArgs a, bool vec, bool pre, bool use_gamma, const GatePlan& plan, hipStream_t stream,
                        int what = kLaunchSlices | kLaunchCombine) {
     a.slices = plan.slices, a.steps_per = plan.steps_per;
+    if (plan.steps_per > 0)  // (the slab launch has set the depth of its own slices)
+        a.err_depth = gate_err_depth(std::min(a.d, plan.steps_per * gate_kc(NBLK, plan.mb)), plan.slices, a.norm_kind);
     const dim3 block(kThreads);
     hipError_t err = hipSuccess;
 #define INFMOE_GATE(M, V, G, P)                                                                                   \
@@ -872,7 +897,9 @@ size_t gate_scratch_floats(int T, int d, int E) {
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids, const float* centroid_stats,
-                            float* scratch, size_t scratch_floats, bool zero_stats, int* nan_flag, int nan_value) {
+                            float* scratch, size_t scratch_floats, bool zero_stats, int* nan_flag, int nan_value,
+                            int* block_hist, bool* block_hist_done) {
+    if (block_hist_done != nullptr) *block_hist_done = false;
     if (T <= 0) return zero_stats && stats ? launch_fill_i32(stats, 4, 0, stream) : hipSuccess;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(centroids) |
                            reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(folded_centroids)) & 15) == 0;
@@ -903,13 +930,17 @@ hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* ce
     const bool use_slab = pre && vec && gate_slab_plan(T, d, E, partial_floats, &slab);
     if (use_slab) {
         // many tokens: partial scores per slice with the centroid slice resident in LDS, then the combine
+        // (one block of tokens: the counting sort does all its passes in one launch and wants no histogram)
+        if (T <= kCountBlockTokens) block_hist = nullptr;
+        const int n_hist = block_hist ? ((T + kCountBlockTokens - 1) / kCountBlockTokens) * E : 0;
         const hipError_t err = launch_gate_slab(slab, T, d, E, x, folded_centroids, scratch, stream,
-                                                zero_stats ? stats : nullptr);
+                                                zero_stats ? stats : nullptr, block_hist, n_hist);
         if (err != hipSuccess) return err;
         plan.mb = T < 64 * kTargetGroups ? 1 : 4;
         plan.groups = (T + 16 * plan.mb - 1) / (16 * plan.mb);
         plan.slices = slab.slices;
         plan.steps_per = 0;  // the combine does not walk the embedding dimension
+        a.err_depth = gate_err_depth(slab.ks, slab.slices, norm_kind);
     } else {
         plan = gate_plan(T, d, E, vec, partial_floats);
         if (zero_stats && stats != nullptr) {
@@ -935,8 +966,12 @@ hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* ce
         }
     }
     if (err != hipSuccess || !lean) return err;
+    if (use_slab && block_hist != nullptr && block_hist_done != nullptr) *block_hist_done = true;
+    const float depth = use_slab ? a.err_depth
+                                 : gate_err_depth(std::min(d, plan.steps_per * gate_kc(nblk_for(E), plan.mb)), plan.slices, norm_kind);
     return launch_gate_combine(T, d, E, plan.slices, scratch, centroid_stats, x, centroids, use_gamma ? gamma : nullptr,
-                               norm_kind, score_bias, sel, coeff, stats, nan_flag, stream, nan_value);
+                               norm_kind, score_bias, sel, coeff, stats, nan_flag, stream, nan_value, depth,
+                               use_slab ? block_hist : nullptr);
 }
 
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats) {

@@ -55,7 +55,8 @@ template <int NBLK, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gate_slab_kernel(const float* __restrict__ X, const float* __restrict__ Cf,
                                                                float* __restrict__ partials, int T, int d, int E,
                                                                int ks, int S, int tiles_per_wave,
-                                                               int* __restrict__ zero_stats) {
+                                                               int* __restrict__ zero_stats,
+                                                               int* __restrict__ zero_hist, int n_hist) {
     extern __shared__ __align__(16) float slab[];  // [16 * NBLK][ks + 4]
     constexpr int EP = 16 * NBLK;
     const int LDK = ks + 4, W = E + 2;
@@ -66,6 +67,9 @@ __global__ __launch_bounds__(64 * WAVES) void gate_slab_kernel(const float* __re
     const size_t k0 = (size_t)j * ks;
     // the routing statistics the combine launch counts into start at zero (saves a fill launch)
     if (zero_stats != nullptr && blockIdx.x == 0 && tid < 4) zero_stats[tid] = 0;
+    // ... and so does the per-block histogram of the assignment that it adds into (saves the histogram launch)
+    if (zero_hist != nullptr)
+        for (int q = blockIdx.x * (64 * WAVES) + tid; q < n_hist; q += gridDim.x * (64 * WAVES)) zero_hist[q] = 0;
 
     // Tiles of this workgroup: (g * tiles_per_wave + it) * WAVES + wave, it = 0 .. tiles_per_wave - 1.
     // The wave walks the chunks of all its tiles as one sequence: chunk n sits in register set n & 1,
@@ -226,6 +230,12 @@ struct CombineArgs {
     int* stats;     // or null
     int* nan_flag;  // null, or an int (host memory the device can write) set to nan_value when a token has no orderable score
     int nan_value;
+    float err_depth;  // n of the error bound of a score (gate_err_depth)
+    // null, or [ceil(T / hist_block)][E] ints, zero on entry, that receive the number of tokens of every block
+    // of hist_block consecutive tokens that chose each expert: what the first pass of the counting sort
+    // (hist_kernel) would compute from sel in a launch of its own
+    int* block_hist;
+    int hist_block;
 };
 
 __device__ __forceinline__ double wave_sum64(double v) {
@@ -241,36 +251,53 @@ constexpr int kCand = 4;  // experts re-scored by one sweep over the embedding d
 // Returns, in every thread, sc[c] = rstd * (x.g.c - mu * sum g.c) + bias for the experts cand[0..kCand).
 // With 256 threads a row of 4096 floats is four float4 per thread, and the unrolled loop has the loads of
 // all rows in flight at once: the sweep costs one memory round trip, not one per piece of the row.
+// NC: how many of the kCand candidates are looked at (2 when only the best two are close, the usual case: half
+// the loads and half the double-precision arithmetic); sc[c] for c >= NC is not set.
+template <int NC>
 __device__ __forceinline__ void rescore(const CombineArgs& a, int t, const int (&cand)[kCand], double (&sc)[kCand],
                                         double (*s_part)[2 + 2 * kCand]) {
     const int tid = threadIdx.x, d = a.d;
     const float* xr = a.X + (size_t)t * d;
-    const float* cr[kCand];
+    const float* cr[NC];
 #pragma unroll
-    for (int c = 0; c < kCand; ++c) cr[c] = a.C + (size_t)cand[c] * d;
+    for (int c = 0; c < NC; ++c) cr[c] = a.C + (size_t)cand[c] * d;
     const bool use_gamma = a.norm_kind != NORM_NONE && a.gamma != nullptr;
+    const bool centered = a.norm_kind == NORM_CENTERED;
     double r[2 + 2 * kCand];
 #pragma unroll
     for (int q = 0; q < 2 + 2 * kCand; ++q) r[q] = 0.0;
-#pragma unroll 4
-    for (int k = 4 * tid; k < d; k += 1024) {
-        const v4f xv = *reinterpret_cast<const v4f*>(xr + k);
-        v4f gv = {1.f, 1.f, 1.f, 1.f};
-        if (use_gamma) gv = *reinterpret_cast<const v4f*>(a.gamma + k);
-        const double x0 = xv.x, x1 = xv.y, x2 = xv.z, x3 = xv.w;
-        r[0] += (x0 + x1) + (x2 + x3);
-        r[1] += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+    // Blocks of 4096 floats, four float4 per thread of each of the six rows: all 24 loads are issued (from
+    // clamped, always valid addresses; a piece beyond the row is masked out of the sums) before the first is
+    // used, so a block costs one trip to memory, not one per piece.  (As a loop with the loads next to their
+    // use the sweep took 11 us of the launch's critical path.)
+    for (int kb = 0; kb < d; kb += 4096) {
+        v4f xv[4], gv[4], cv[NC][4];
 #pragma unroll
-        for (int c = 0; c < kCand; ++c) {
-            const v4f cv = *reinterpret_cast<const v4f*>(cr[c] + k);
-            const double g0 = (double)gv.x * (double)cv.x, g1 = (double)gv.y * (double)cv.y;
-            const double g2 = (double)gv.z * (double)cv.z, g3 = (double)gv.w * (double)cv.w;
-            r[2 + c] += (x0 * g0 + x1 * g1) + (x2 * g2 + x3 * g3);
-            r[2 + kCand + c] += (g0 + g1) + (g2 + g3);
+        for (int u = 0; u < 4; ++u) {
+            const int k = min(kb + 1024 * u + 4 * tid, d - 4);
+            xv[u] = *reinterpret_cast<const v4f*>(xr + k);
+            gv[u] = use_gamma ? *reinterpret_cast<const v4f*>(a.gamma + k) : v4f{1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c) cv[c][u] = *reinterpret_cast<const v4f*>(cr[c] + k);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (kb + 1024 * u + 4 * tid >= d) continue;
+            const double x0 = xv[u].x, x1 = xv[u].y, x2 = xv[u].z, x3 = xv[u].w;
+            r[0] += (x0 + x1) + (x2 + x3);
+            r[1] += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const double g0 = (double)gv[u].x * (double)cv[c][u].x, g1 = (double)gv[u].y * (double)cv[c][u].y;
+                const double g2 = (double)gv[u].z * (double)cv[c][u].z, g3 = (double)gv[u].w * (double)cv[c][u].w;
+                r[2 + c] += (x0 * g0 + x1 * g1) + (x2 * g2 + x3 * g3);
+                if (centered) r[2 + kCand + c] += (g0 + g1) + (g2 + g3);  // (only the centered norm wants sum g c)
+            }
         }
     }
 #pragma unroll
     for (int q = 0; q < 2 + 2 * kCand; ++q) {
+        if ((q >= 2 + NC && q < 2 + kCand) || q >= 2 + kCand + NC) continue;  // sums of candidates not looked at
         r[q] = wave_sum64(r[q]);
         if ((tid & 63) == 0) s_part[tid >> 6][q] = r[q];
     }
@@ -286,7 +313,7 @@ __device__ __forceinline__ void rescore(const CombineArgs& a, int t, const int (
         rstd = 1.0 / sqrt(fmax(r[1] / d - mu * mu, 0.0) + 1e-6);
     }
 #pragma unroll
-    for (int c = 0; c < kCand; ++c) {
+    for (int c = 0; c < NC; ++c) {
         sc[c] = rstd * (r[2 + c] - mu * r[2 + kCand + c]);
         if (a.bias != nullptr) sc[c] += (double)a.bias[cand[c]];
     }
@@ -362,10 +389,12 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
 #pragma unroll
     for (int off = 8; off > 0; off >>= 1) second = fmaxf(second, __shfl_xor(second, off));
 
-    // FP32 accumulation over d terms cannot order two scores closer than its own rounding error
-    const float bound = 8.f * FLT_EPSILON * rstd * sqrtf(a2) * cnmax;
+    // FP32 accumulation over d terms cannot order two scores closer than twice its own rounding error (gate_err_depth)
+    const float bound = a.err_depth * FLT_EPSILON * rstd * sqrtf(a2) * cnmax;
     const float thr = fmaxf(bound, 4e-6f * fabsf(best));
     const bool flagged = live && besti >= 0 && E > 1 && (best - second) < thr;
+    __shared__ int s_sel[16];  // the 16 tokens' experts, as last decided
+    if (i == 0) s_sel[threadIdx.x >> 4] = live ? max(besti, 0) : -1;
     if (live && i == 0) {
         a.sel[t] = besti < 0 ? 0 : besti;  // no orderable score: the reference asserts (plugin/cuda/moe.cu:70)
         a.coeff[t] = besti < 0 ? __builtin_nanf("") : best;  // NaN marks the row: the combine step writes NaN for it
@@ -426,8 +455,12 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
                 }
             };
             double sc[kCand];
-            if (nc <= kCand) {
-                rescore(a, tt, cand, sc, s_part);
+            if (nc <= 2) {
+                rescore<2>(a, tt, cand, sc, s_part);
+                offer(sc[0], cand[0]);
+                if (nc == 2) offer(sc[1], cand[1]);
+            } else if (nc <= kCand) {
+                rescore<kCand>(a, tt, cand, sc, s_part);
 #pragma unroll
                 for (int c = 0; c < kCand; ++c)
                     if (c < nc) offer(sc[c], cand[c]);
@@ -435,7 +468,7 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
                 for (int e0 = 0; e0 < E; e0 += kCand) {
 #pragma unroll
                     for (int c = 0; c < kCand; ++c) cand[c] = min(e0 + c, E - 1);
-                    rescore(a, tt, cand, sc, s_part);
+                    rescore<kCand>(a, tt, cand, sc, s_part);
 #pragma unroll
                     for (int c = 0; c < kCand; ++c)
                         if (e0 + c < E) offer(sc[c], e0 + c);
@@ -445,6 +478,7 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
                 if (topi >= 0) {
                     a.sel[tt] = topi;
                     a.coeff[tt] = (float)top;
+                    s_sel[tt - blockIdx.x * 16] = topi;
                 }
                 if (a.stats != nullptr) {
                     atomicAdd(&a.stats[2], 1);
@@ -454,16 +488,22 @@ __global__ __launch_bounds__(256) void gate_combine_kernel(const CombineArgs a) 
             // rescore() ends with a barrier, so s_cand / s_nc may be rewritten by the next token's owner
         }
     }
+    if (a.block_hist != nullptr) {  // integer sums: the order the additions arrive in does not matter
+        __syncthreads();
+        const int tk = blockIdx.x * 16 + threadIdx.x;
+        if (threadIdx.x < 16 && s_sel[threadIdx.x] >= 0)
+            atomicAdd(&a.block_hist[(size_t)(tk / a.hist_block) * E + s_sel[threadIdx.x]], 1);
+    }
 }
 
 template <int NBLK, int WAVES>
 hipError_t launch_one(const GateSlabPlan& p, int T, int d, int E, const float* x, const float* cf, float* partials,
-                      int* zero_stats, hipStream_t stream) {
+                      int* zero_stats, int* zero_hist, int n_hist, hipStream_t stream) {
     const size_t lds = (size_t)16 * NBLK * (p.ks + 4) * sizeof(float);
     const hipError_t err = allow_lds_once<gate_slab_kernel<NBLK, WAVES>>(kSlabLdsLimit);
     if (err != hipSuccess) return err;
     gate_slab_kernel<NBLK, WAVES><<<dim3(p.groups * p.slices), 64 * WAVES, lds, stream>>>(x, cf, partials, T, d, E, p.ks,
-                                                                                         p.slices, p.tiles_per_wave, zero_stats);
+                                                                                         p.slices, p.tiles_per_wave, zero_stats, zero_hist, n_hist);
     return hipGetLastError();
 }
 
@@ -526,16 +566,16 @@ size_t gate_slab_scratch_floats(int T, int d, int E) {
 }
 
 hipError_t launch_gate_slab(const GateSlabPlan& p, int T, int d, int E, const float* x, const float* folded_centroids,
-                            float* partials, hipStream_t stream, int* zero_stats) {
+                            float* partials, hipStream_t stream, int* zero_stats, int* zero_hist, int n_hist) {
     if (p.ks < kChunk || (p.ks & (p.ks - 1)) != 0 || p.slices * p.ks != d || p.groups <= 0 || p.tiles_per_wave <= 0)
         return hipErrorInvalidValue;
     if ((long long)p.groups * p.tiles_per_wave * p.waves * 16 < T) return hipErrorInvalidValue;  // tokens not covered
     if ((size_t)16 * nblk_of(E) * (p.ks + 4) * sizeof(float) > kSlabLdsLimit) return hipErrorInvalidValue;
     if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(folded_centroids)) & 15) != 0) return hipErrorInvalidValue;
 #define INFMOE_SLAB(NB)                                                                                     \
-    return p.waves == 8 ? launch_one<NB, 8>(p, T, d, E, x, folded_centroids, partials, zero_stats, stream)              \
-                        : (p.waves == 4 ? launch_one<NB, 4>(p, T, d, E, x, folded_centroids, partials, zero_stats, stream) \
-                                        : hipErrorInvalidValue)
+    return p.waves == 8 ? launch_one<NB, 8>(p, T, d, E, x, folded_centroids, partials, zero_stats, zero_hist, n_hist, stream) \
+           : (p.waves == 4 ? launch_one<NB, 4>(p, T, d, E, x, folded_centroids, partials, zero_stats, zero_hist, n_hist, stream) \
+                           : hipErrorInvalidValue)
     switch (nblk_of(E)) {
         case 1: INFMOE_SLAB(1);
         case 2: INFMOE_SLAB(2);
@@ -555,13 +595,14 @@ bool gate_combine_ok(int d, int E) { return E <= 128 && d % 4 == 0; }
 hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* partials, const float* centroid_stats,
                                const float* x, const float* centroids, const float* gamma, int norm_kind,
                                const float* score_bias, int* sel, float* coeff, int* stats, int* nan_flag,
-                               hipStream_t stream, int nan_value) {
+                               hipStream_t stream, int nan_value, float err_depth, int* block_hist) {
     if (T <= 0) return hipSuccess;
     if (!gate_combine_ok(d, E) || slices < 1 || slices > kGateMaxSlices) return hipErrorInvalidValue;
     CombineArgs a{};
     a.T = T, a.d = d, a.E = E, a.S = slices;
     a.partials = partials, a.cstats = centroid_stats, a.X = x, a.C = centroids, a.gamma = gamma, a.bias = score_bias;
-    a.norm_kind = norm_kind, a.sel = sel, a.coeff = coeff, a.stats = stats, a.nan_flag = nan_flag, a.nan_value = nan_value;
+    a.norm_kind = norm_kind, a.sel = sel, a.coeff = coeff, a.stats = stats, a.nan_flag = nan_flag, a.nan_value = nan_value, a.err_depth = err_depth;
+    a.block_hist = block_hist, a.hist_block = kCountBlockTokens;
     const dim3 grid((T + 15) / 16);
     switch (nblk_of(E)) {
         case 1: gate_combine_kernel<1><<<grid, 256, 0, stream>>>(a); break;

@@ -31,13 +31,16 @@ constexpr float kNormEps = 1e-6f;  // plugin/MoELayerPlugin.cc:324, plugin/subla
 // A token without an orderable score (a NaN in its row; the reference asserts, plugin/cuda/moe.cu:70) gets
 // expert 0 and the coefficient NaN, is counted in stats[1], and sets *nan_flag (an int the device can
 // write, e.g. page-locked host memory) to nan_value (say, a number that names the call) when that pointer is given.
+// Optional: block_hist, the scratch of launch_expert_count for the same T and E.  A call that takes the two-launch
+// path for many tokens leaves the first pass of the counting sort in it (tokens per expert of every block of
+// kCountBlockTokens tokens) and sets *block_hist_done; launch_expert_count is then told to skip that pass.
 size_t gate_scratch_floats(int T, int d, int E);
 hipError_t launch_gate_top1(int T, int d, int E, const float* x, const float* centroids, const float* gamma,
                             int norm_kind, const float* score_bias, int* sel, float* coeff, int* stats,
                             hipStream_t stream, const float* folded_centroids = nullptr,
                             const float* centroid_stats = nullptr, float* scratch = nullptr,
                             size_t scratch_floats = 0, bool zero_stats = false, int* nan_flag = nullptr,
-                            int nan_value = 1);
+                            int nan_value = 1, int* block_hist = nullptr, bool* block_hist_done = nullptr);
 // Calls with many tokens: the first of two launches writes partial scores per slice of the embedding
 // dimension with that slice of the folded centroids resident in LDS (gating_slab.hip); the combine launch
 // of the gating kernel adds the slices and selects.  The plan says how a call is cut; gate_slab_plan
@@ -56,9 +59,10 @@ bool gate_slab_plan(int T, int d, int E, size_t scratch_floats, GateSlabPlan* pl
 size_t gate_slab_scratch_floats(int T, int d, int E);
 // partials: [slices][T][E + 2] floats (dot products, row sum, row sum of squares)
 // zero_stats: null, or 4 ints that the launch sets to zero (the combine launch counts into them)
+// zero_hist: null, or n_hist ints that the launch sets to zero (the block histogram the combine launch adds into)
 hipError_t launch_gate_slab(const GateSlabPlan& plan, int T, int d, int E, const float* x,
                             const float* folded_centroids, float* partials, hipStream_t stream,
-                            int* zero_stats = nullptr);
+                            int* zero_stats = nullptr, int* zero_hist = nullptr, int n_hist = 0);
 // The second launch of a sliced gating call: adds the slices' partial scores ([slices][T][E + 2]), selects,
 // and re-scores near ties in float64 from x, the plain centroids and gamma.  Takes up to 128 experts and
 // rows of 16-byte-aligned float4 (gate_combine_ok); centroid_stats as fold_centroids_host makes them.
@@ -66,7 +70,11 @@ bool gate_combine_ok(int d, int E);
 hipError_t launch_gate_combine(int T, int d, int E, int slices, const float* partials, const float* centroid_stats,
                                const float* x, const float* centroids, const float* gamma, int norm_kind,
                                const float* score_bias, int* sel, float* coeff, int* stats, int* nan_flag,
-                               hipStream_t stream, int nan_value = 1);
+                               hipStream_t stream, int nan_value, float err_depth, int* block_hist = nullptr);
+// n of the rounding-error bound n * FLT_EPSILON * rstd * |x| * max|g c| under which two FP32 scores are not
+// trusted to be in the exact order (such a token is re-scored in float64): slices of `slice_floats` floats of the
+// embedding dimension, `slices` of them.
+float gate_err_depth(int slice_floats, int slices, int norm_kind);
 void fold_centroids_host(int d, int E, const float* centroids, const float* gamma, float* folded, float* cstats);
 
 // ---- dispatch (replaces moe_expert_count, plugin/cuda/moe.cu:161-212)
@@ -99,9 +107,10 @@ inline int xcd_tile_capacity(int max_tiles) {
 //     over the experts with more than `skinny_max` rows, dealt to the 8 XCDs so that the padded
 //     row counts balance, each XCD's share in descending height
 //   row_expert[T]: expert of every routed row
+// hist_ready: the scratch already holds the per-block histogram of sel (launch_gate_top1 left it there).
 hipError_t launch_expert_count(int T, int E, const int* sel, int* pos, int* count, int* offset, void* scratch,
                                RowTile* tiles, int* sched, int tile_rows, int skinny_max, int* row_expert,
-                               hipStream_t stream);
+                               hipStream_t stream, bool hist_ready = false);
 
 // The same with the scratch in a device array owned by the library (kExpertCountStaticInts ints per GPU,
 // held until the process ends): no allocation and no caller-supplied scratch.  Calls on one GPU share
@@ -201,8 +210,9 @@ inline bool gemm_small_tiles(int tokens, int experts, int ffn_kind) {
     return ffn_kind != FFN_GATED_GELU && (long long)tokens <= 64ll * experts;
 }
 
-// Few-row experts (decode): every weight row is streamed once and dotted with up to
-// kSkinnyMaxRows activation rows held in LDS.
+// Few-row experts (decode): every weight row is streamed once and dotted with up to kSkinnyMaxRows activation
+// rows held in registers; an expert with more rows is done in runs of kSkinnyMaxRows, one pass over its weights
+// each.
 constexpr int kSkinnyMaxRows = 8;
 hipError_t launch_expert_skinny(const GemmProblem& p, int rows, hipStream_t stream);
 hipError_t launch_expert_skinny_grouped(const GemmProblem& p, size_t weight_stride, const int* count,

@@ -360,10 +360,11 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     INFMOE_TRY(mark(0));
     // 0-2. norm (cpm_2: for scoring only), scores, top-1          plugin/MoELayerPlugin.cc:312-345
     const bool ln = mParams.flags.layernormOnInputBeforeScore;
+    bool histReady = false;  // the gating leaves the first pass of the counting sort behind when it can
     INFMOE_HIP(launch_gate_top1(T, d, E, x, mCentroidsGpu, ln ? mLayernormGpu : nullptr, ln ? mParams.normKind : NORM_NONE,
                                 mScoreBias.empty() ? nullptr : mScoreBiasGpu, c.sel, c.coeff, dStats, stream, mFoldedGpu,
                                 mFoldedGpu + (size_t)E * d, c.gateScratch, gate_scratch_floats(T, d, E),
-                                /*zero_stats=*/true, mNanFlagDev, mCallNumber));
+                                /*zero_stats=*/true, mNanFlagDev, mCallNumber, static_cast<int*>(c.countScratch), &histReady));
     INFMOE_TRY(mark(1));
     // 3. count, sort, scatter                                      plugin/MoELayerPlugin.cc:349-355
     // (the row tiles of the grouped expert launch are made on either schedule: streamed experts that are all
@@ -371,7 +372,7 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     const bool grouped = resident();
     const int skinnyMax = mSublayer->skinnyMaxRows(T);
     INFMOE_HIP(launch_expert_count(T, E, c.sel, c.pos, dCount, dOffset, c.countScratch, c.tiles, c.sched,
-                                   mSublayer->rowTileHeightFor(T), skinnyMax, c.rowExpert, stream));
+                                   mSublayer->rowTileHeightFor(T), skinnyMax, c.rowExpert, stream, histReady));
     INFMOE_TRY(mark(2));
     // experts see the raw input (:354); the statistics of their row norm are taken while the rows are copied
     INFMOE_HIP(launch_scatter(T, d, x, c.coeff, c.pos, c.routed, c.routedCoeff, stream, c.rowStats, mSublayer->rowStatsKind()));

@@ -198,9 +198,11 @@ Status T5FFLayer::copyWeights(void* dst, int expert, hipStream_t stream) {
 // two workgroups per compute unit, streams the weights faster than the few-row kernel and one more launch
 // would: 128 tokens over 32 experts of 4096 x 10240 take 0.80 ms per launch against 0.95 ms.)
 static bool decode_like(int layerTokens, int expertCount) { return layerTokens <= 2 * expertCount; }
+constexpr int kAllRows = 1 << 30;
 
 int T5FFLayer::skinnyMaxRows(int32_t tokenCount) const {
-    return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kSkinnyMaxRows : 0;
+    // (every expert of a decode call, whatever its rows: the few-row kernel takes a taller one in runs of 8)
+    return decode_like(tokenCount, mExpertCount) && mEmbeddingSize % 4 == 0 && mHiddenSize % 4 == 0 ? kAllRows : 0;
 }
 
 // folded (rms norm only): `weights` is a slot as copyWeights leaves it (gamma multiplied into the input-side
@@ -237,7 +239,7 @@ Status T5FFLayer::runOne(int rows, int layerTokens, int expertCount, int d, int 
     g2.A = hid, g2.B = w + d + (size_t)(nMat - 1) * dh, g2.R = in, g2.C = out, g2.N = d, g2.K = h;
     g2.epilogue = EPI_RESIDUAL;
     const bool aligned = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(g1.A) | reinterpret_cast<uintptr_t>(hid)) & 15) == 0;
-    const bool skinny = rows <= kSkinnyMaxRows && decode_like(layerTokens, expertCount) && d % 4 == 0 && h % 4 == 0 && aligned;
+    const bool skinny = decode_like(layerTokens, expertCount) && d % 4 == 0 && h % 4 == 0 && aligned;
     if (skinny) {
         INFMOE_HIP(launch_expert_skinny(g1, rows, stream));
         INFMOE_HIP(launch_expert_skinny(g2, rows, stream));
@@ -300,6 +302,12 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
     const bool skinny = skinnyMaxRows(T) > 0;
     g1.small_tiles = g2.small_tiles = gemm_small_tiles(T, mExpertCount, mFfnKind) ? 1 : 0;
     if (g.afterNorm) INFMOE_HIP(hipEventRecord(g.afterNorm, g.stream));
+    if (skinny) {  // a decode call: every expert through the few-row kernel (as runOne does for it)
+        INFMOE_HIP(launch_expert_skinny_grouped(g1, stride, g.count, g.offset, mExpertCount, g.stream));
+        if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, g.stream));
+        INFMOE_HIP(launch_expert_skinny_grouped(g2, stride, g.count, g.offset, mExpertCount, g.stream));
+        return INFMOE_OK;
+    }
     if (!expert_gemm_grouped_ok(g1, stride) || !expert_gemm_grouped_ok(g2, stride)) {
         // sizes the matrix-core kernel does not take (d or h not a multiple of 32)
         INFMOE_HIP(launch_expert_gemm_any_shape_grouped(g1, stride, g.rowExpert, T, g.stream));
@@ -308,10 +316,8 @@ Status T5FFLayer::runGrouped(const GroupedRun& g) {
         return INFMOE_OK;
     }
     INFMOE_HIP(launch_expert_gemm_grouped(g1, stride, g.tiles, g.sched, g.maxTiles, g.stream));
-    if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g1, stride, g.count, g.offset, mExpertCount, g.stream));
     if (g.afterGemm1) INFMOE_HIP(hipEventRecord(g.afterGemm1, g.stream));
     INFMOE_HIP(launch_expert_gemm_grouped(g2, stride, g.tiles, g.sched, g.maxTiles, g.stream));
-    if (skinny) INFMOE_HIP(launch_expert_skinny_grouped(g2, stride, g.count, g.offset, mExpertCount, g.stream));
     return INFMOE_OK;
 }
 
