@@ -61,7 +61,7 @@ struct RowTile {
     int32_t expert;
     int32_t row0; /* first routed row */
     int32_t rows; /* 1..tile height */
-    int32_t pad;
+    int32_t pad;  /* place in its run | length of the run << 16 (a run: row tiles of one expert scheduled together); 0: by itself */
 };
 
 /* Everything a sub-layer needs to run every expert of one layer call from a single set of launches. */

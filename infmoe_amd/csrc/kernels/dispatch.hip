@@ -48,6 +48,7 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(int T, int E, const int*
 }
 
 constexpr int kMaxSortedTiles = 1024;  // row tiles the scan orders by cost; beyond that they stay in expert order
+constexpr int kRunTiles = 4;           // row tiles of one expert that share their weight tiles through an XCD's L2
 
 // `tiles` holds 2*max_tiles entries (the second half is spare), `sched` kSchedInts ints:
 // [0] number of row tiles, [1 + x] first tile of XCD x (x = 0..8).
@@ -99,16 +100,28 @@ __device__ __forceinline__ void scan_body(int T, int E, int nblk, int* __restric
         if (c <= skinny_max) continue;
         int j = s_tile0[e];
         const int per = row_tile_height(c, tile_rows);
+        // (runs: see below; an expert's nt tiles make as few runs as kRunTiles allows, of equal length)
+        const int nt = (c + tile_rows - 1) / tile_rows, nruns = (nt + kRunTiles - 1) / kRunTiles;
+        const int len = (nt + nruns - 1) / nruns;
+        int p = 0, head = j, cost = 0;
         for (int m0 = 0; m0 < c; m0 += per, ++j) {
             RowTile rt;
             rt.expert = e;
             rt.row0 = s_off[e] + m0;
             rt.rows = min(per, c - m0);
             rt.pad = 0;
-            if (sorted)
+            if (sorted) {
+                rt.pad = p | (min(len, nt - (head - s_tile0[e])) << 16);  // place in the run | length of the run
                 s_raw[j] = rt;
-            else
+                s_cost[j] = -1;  // not the head of a run (the head's entry is set when the run is complete)
+                cost += (rt.rows + 15) >> 4;
+                if (++p == len || m0 + per >= c) {
+                    s_cost[head] = cost;  // a run is known by its first tile; its cost: the padded height of its tiles
+                    p = 0, head = j + 1, cost = 0;
+                }
+            } else {
                 tiles[j] = rt;  // many tiles balance by themselves: expert order, equal contiguous shares
+            }
         }
     }
     if (!sorted) {
@@ -116,38 +129,77 @@ __device__ __forceinline__ void scan_body(int T, int E, int nblk, int* __restric
         if (threadIdx.x == 0) sched[0] = n;
         return;
     }
+    __shared__ int s_nruns;
+    if (threadIdx.x == 0) s_nruns = 0;  // (no tiles at all: nobody counts the runs below)
     __syncthreads();
-    // Balance the 8 XCDs: order the tiles by padded height (the cost of a tile) and deal them out in
-    // snake order (XCD 0..7, then 7..0, ...), which keeps the loads within one tile of each other and,
-    // unlike a greedy assignment, lets every tile compute its own place.  Inside an XCD the order
-    // stays descending, so the short tiles fill the tail.
-    for (int j = threadIdx.x; j < n; j += kThreads) s_cost[j] = (s_raw[j].rows + 15) >> 4;
-    __syncthreads();
-    const int full = n / kXcdCount, rem = n % kXcdCount;
-    auto share = [&](int x) {  // tiles of XCD x: one per full round plus its part of the last, partial round
-        const bool extra = (full & 1) == 0 ? x < rem : x >= kXcdCount - rem;
-        return full + (extra ? 1 : 0);
-    };
-    if (threadIdx.x == 0) {
-        int start = 0;
-        s_sched[0] = n;
-        for (int x = 0; x < kXcdCount; ++x) {
-            s_sched[1 + x] = start;
-            start += share(x);
+    // Runs.  The row tiles of an expert with several of them (all of one height but the last) are kept together
+    // in runs of up to kRunTiles: a run goes to one XCD as a whole, and the launch takes its workgroups column tile
+    // by column tile, the run's row tiles side by side, so that workgroups that start together read the same
+    // weight rows and all but one find them in the XCD's L2.  (Tile by tile, an expert of 19 row tiles had its
+    // weights fetched from memory 19 times.)  An expert's tiles are cut into as few runs as kRunTiles allows, of
+    // equal length (made with the tiles, above); a run is the unit of the balance below.
+    // Heaviest run first to the XCD with the least work so far (among those with room: the grid is sized for
+    // xcd_cap tiles per XCD).  Inside an XCD the runs keep that order, so the light ones fill the tail.  The
+    // assignment is sequential by nature; it is done by one wave whose lanes 0..7 each keep one XCD's work and
+    // tile count in registers, 64 runs fetched from LDS at a time, the minimum found with three lane
+    // exchanges inside the registers (one thread walking LDS took 0.3 us per run).
+    __shared__ int s_order[kMaxSortedTiles];   // heads of runs by descending cost
+    __shared__ int s_place[kMaxSortedTiles];   // per head: XCD << 16 | position inside the XCD's share
+    for (int j = threadIdx.x; j < n; j += kThreads) {
+        const int cj = s_cost[j];
+        int rank = 0, heads = 0;
+        for (int i = 0; i < n; ++i) {
+            const int ci = s_cost[i];
+            rank += (ci > cj) || (ci == cj && i < j);
+            heads += ci >= 0;
         }
-        s_sched[1 + kXcdCount] = start;
+        if (cj >= 0) s_order[rank] = j;
+        if (j == 0) s_nruns = heads;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        static_assert(kXcdCount == 8, "the minimum below is taken over eight lanes");
+        const int lane = threadIdx.x;
+        int load = 0, held = 0;  // lanes 0..7: work (padded 16-row units) and row tiles given to XCD `lane` so far
+        const int nruns = s_nruns;
+        auto lane_min = [](int v) {  // the minimum over each group of eight lanes, in all of them
+            v = min(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));   // lane ^ 1
+            v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));   // lane ^ 2
+            return min(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));  // lane <-> 7 - lane
+        };
+        for (int r0 = 0; r0 < nruns; r0 += 64) {
+            const int mine = r0 + lane < nruns ? s_order[r0 + lane] : 0;  // lane q: run r0 + q
+            const int my_len = s_raw[mine].pad >> 16, my_cost = s_cost[mine];
+            const int cnt = min(64, nruns - r0);
+            for (int q = 0; q < cnt; ++q) {
+                const int head = __builtin_amdgcn_readlane(mine, q), L = __builtin_amdgcn_readlane(my_len, q);
+                const int cost = __builtin_amdgcn_readlane(my_cost, q);
+                // (work << 3 | lane: the least work wins, the lower XCD on a tie; work stays far below 2^27)
+                const int key = lane < kXcdCount && held + L <= xcd_cap ? (load << 3) | lane : 0x7fffffff;
+                const int won = __builtin_amdgcn_readfirstlane(lane_min(key));
+                // (no XCD with room cannot happen: the capacities add up to more than twice the tiles)
+                const int best = won == 0x7fffffff ? 0 : won & 7;
+                if (lane == best) {
+                    s_place[head] = (best << 16) | held;
+                    load += cost;
+                    held += L;
+                }
+            }
+        }
+        int start = 0;
+        for (int x = 0; x < kXcdCount; ++x) {
+            if (lane == 0) s_sched[1 + x] = start;
+            start += __builtin_amdgcn_readlane(held, x);
+        }
+        if (lane == 0) s_sched[1 + kXcdCount] = start, s_sched[0] = n;
     }
     __syncthreads();
     for (int j = threadIdx.x; j < n; j += kThreads) {
-        const int cj = s_cost[j];
-        int rank = 0;
-        for (int i = 0; i < n; ++i) rank += (s_cost[i] > cj) || (s_cost[i] == cj && i < j);
-        const int round = rank / kXcdCount, idx = rank % kXcdCount;
-        const int x = (round & 1) == 0 ? idx : kXcdCount - 1 - idx;
-        tiles[s_sched[1 + x] + round] = s_raw[j];
+        const int p = s_raw[j].pad & 0xffff, head = j - p;
+        const int place = s_place[head];
+        tiles[s_sched[1 + (place >> 16)] + (place & 0xffff) + p] = s_raw[j];
     }
     if (threadIdx.x < 2 + kXcdCount) sched[threadIdx.x] = s_sched[threadIdx.x];
-    (void)xcd_cap;  // a share never exceeds ceil(n / 8), which is below the capacity the grid was sized for
     (void)T;
     (void)max_tiles;
 }

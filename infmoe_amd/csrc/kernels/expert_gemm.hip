@@ -100,7 +100,7 @@ hipError_t launch_expert_gemm(const GemmProblem& p, int rows, int tile_rows, hip
     }
     const int tile = std::min(row_tile_height(rows, tile_rows), ((rows + 15) / 16) * 16);
     const int a_alloc = ((tile + 31) / 32) * 32;  // whole 32-row slabs
-    const dim3 grid((p.N + kGemmColumns - 1) / kGemmColumns, (rows + tile - 1) / tile);
+    const dim3 grid((rows + tile - 1) / tile, (p.N + kGemmColumns - 1) / kGemmColumns);  // x: row tiles, y: column tiles
     if (p.small_tiles) {
         // (LDS for the tallest tile of this form whatever this expert's height: the two-workgroups-per-unit
         // residency is the same for every launch of the form)

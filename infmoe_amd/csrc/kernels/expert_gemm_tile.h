@@ -81,7 +81,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 // normed rows with the plain weights (stats: [row][2], of which [1] = rstd_r is used).  The inner loop does
 // not know of any of it.
 // D: register sets of the global loads, i.e. how many K steps they run ahead of the matrix core (2 or 4).
-template <int NMB, int G4, int BN, int EPI, int BK, int D>
+template <int NMB, int G4, int BN, int EPI, int BK, int D, bool STREAM_B = false>
 __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const float* __restrict__ R,
                                           float* __restrict__ C, int rows, const float* __restrict__ B0,
                                           const float* __restrict__ B1, int n0, int N, int K,
@@ -157,10 +157,12 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             ra[P][L] = *reinterpret_cast<const v4f*>(a_base + (size_t)k0 * 4 + a_off[L]);
         } else {
             constexpr int M = (L - A_LOADS) / B_LOADS, Q = (L - A_LOADS) % B_LOADS;
-            // a weight byte is read by one workgroup, once (by a few where an expert has several row tiles):
-            // streamed past the caches.  With few rows per expert, where the weights' arrival sets the pace, that
-            // is worth 3-6 % (256-512 tokens over 32 experts); with many it changes nothing.
-            rb[P][M][Q] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(b_base[M] + (size_t)k0 * 4 + b_off[Q]));
+            // STREAM_B (calls with few rows per expert): a weight byte is read by one workgroup, once: streamed past
+            // the caches, which is worth 3-6 % where the weights' arrival sets the pace (256-512 tokens over 32
+            // experts).  Tall tiles: plain loads - the row tiles of an expert with several are scheduled side by
+            // side to share their weight rows through the L2, and a line marked as streaming does not stay for that.
+            const v4f* src = reinterpret_cast<const v4f*>(b_base[M] + (size_t)k0 * 4 + b_off[Q]);
+            rb[P][M][Q] = STREAM_B ? __builtin_nontemporal_load(src) : *src;
         }
     };
     // item L of register set P into LDS buffer BUF
@@ -469,33 +471,52 @@ __device__ __forceinline__ void gemm_dispatch(const float* A, const float* R, fl
 #undef INFMOE_CASE_G
 }
 
-// One expert: grid.x = column tiles, grid.y = row tiles of tile_rows rows (the last may be shorter).
+// One expert: grid.x = row tiles of tile_rows rows (the last may be shorter), grid.y = column tiles: the row tiles
+// of a column tile are dispatched side by side and share its weight rows through the caches.
 template <int BN, int EPI>
 __global__ __launch_bounds__(kThreads) void expert_gemm_kernel(GemmProblem p, int rows_total, int tile_rows,
                                                                int a_alloc_rows) {
     extern __shared__ __align__(16) float smem[];
-    const int row0 = blockIdx.y * tile_rows;
+    const int row0 = blockIdx.x * tile_rows;
     const int rows = min(tile_rows, rows_total - row0);
-    const int n0 = blockIdx.x * BN;
+    const int n0 = blockIdx.y * BN;
     gemm_dispatch<BN, EPI>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
                            p.C + (size_t)row0 * p.N, rows, p.B, p.B1, n0, p.N, p.K,
                            p.row_stats ? p.row_stats + 2 * (size_t)row0 : nullptr, smem, a_alloc_rows);
 }
 
 // All experts: 1-D grid of 8 * (row-tile capacity of an XCD) * n_col_tiles workgroups.  Workgroup id
-// b runs on XCD b % 8 and takes slot b / 8 of that XCD's share of the schedule: the share's row
-// tiles in descending height, all column tiles of a row tile in a row (they share its activations).
+// b runs on XCD b % 8 and takes slot b / 8 of that XCD's share of the schedule.  The share is a list of runs
+// of row tiles (RowTile::pad = place in the run | run length << 16; a run is 1..4 row tiles of one expert, the
+// dispatch scan makes them): a run of L tiles owns L * n_col_tiles consecutive slots, column tile by column
+// tile with the run's L row tiles side by side, so workgroups that start together read the same weight rows
+// (one fetch from memory, L - 1 hits in the XCD's L2) and the column tiles of a row tile, which share its
+// activations, follow each other at a distance of L.
+// Returns false for a slot beyond the share.
+__device__ __forceinline__ bool grouped_slot(const RowTile* __restrict__ tiles, const int* __restrict__ sched,
+                                             int n_col_tiles, RowTile* rt, int* col_tile) {
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
+    if (slot >= share * n_col_tiles) return false;
+    const int i = slot / n_col_tiles;  // some tile of the run the slot belongs to
+    const int pad = tiles[first + i].pad;
+    const int L = max(pad >> 16, 1), i0 = i - (pad & 0xffff);
+    const int local = slot - i0 * n_col_tiles;
+    *rt = tiles[first + i0 + local % L];
+    *col_tile = local / L;
+    return true;
+}
+
 template <int BN, int EPI>
 __global__ __launch_bounds__(kThreads) void expert_gemm_grouped_kernel(GemmProblem p, size_t weight_stride,
                                                                        const RowTile* __restrict__ tiles,
                                                                        const int* __restrict__ sched,
                                                                        int n_col_tiles) {
     extern __shared__ __align__(16) float smem[];
-    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
-    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
-    if (slot >= share * n_col_tiles) return;
-    const RowTile rt = tiles[first + slot / n_col_tiles];
-    const int n0 = (slot % n_col_tiles) * BN;
+    RowTile rt;
+    int col_tile;
+    if (!grouped_slot(tiles, sched, n_col_tiles, &rt, &col_tile)) return;
+    const int n0 = col_tile * BN;
     const int owner = p.expert_slot ? p.expert_slot[rt.expert] : rt.expert;
     constexpr bool GATED = EPI == EPI_GATED_GELU;
     const float* B0 = p.B + (size_t)owner * weight_stride;
@@ -528,8 +549,8 @@ __device__ __forceinline__ void gemm_dispatch_small(const float* A, const float*
 #define INFMOE_SMALL_G(n, g)                                                                                          \
     case 4 * (n) + (g):                                                                                               \
         if constexpr ((n) <= kMaxMb && ((g) == 0 || ((n) >= 2 && (n) < kMaxMb)))                                      \
-            gemm_tile<n, g, BN, EPI, 32, depth_of(n, g)>(A, R, C, rows, B0, nullptr, n0, N, K, stats, smem,           \
-                                                         a_alloc_rows);                                              \
+            gemm_tile<n, g, BN, EPI, 32, depth_of(n, g), true>(A, R, C, rows, B0, nullptr, n0, N, K, stats, smem,     \
+                                                               a_alloc_rows);                                        \
         break;
 #define INFMOE_SMALL(n) INFMOE_SMALL_G(n, 0) INFMOE_SMALL_G(n, 1) INFMOE_SMALL_G(n, 2)
     switch (4 * nmb + g4) {
@@ -544,9 +565,9 @@ template <int BN, int EPI>
 __global__ __launch_bounds__(kThreads, 2) void expert_gemm_small_kernel(GemmProblem p, int rows_total, int tile_rows,
                                                                         int a_alloc_rows) {
     extern __shared__ __align__(16) float smem[];
-    const int row0 = blockIdx.y * tile_rows;
+    const int row0 = blockIdx.x * tile_rows;  // (x = row tile, y = column tile, as in expert_gemm_kernel)
     const int rows = min(tile_rows, rows_total - row0);
-    const int n0 = blockIdx.x * BN;
+    const int n0 = blockIdx.y * BN;
     gemm_dispatch_small<BN, EPI>(p.A + (size_t)row0 * p.K, p.R ? p.R + (size_t)row0 * p.N : nullptr,
                                  p.C + (size_t)row0 * p.N, rows, p.B, n0, p.N, p.K,
                                  p.row_stats ? p.row_stats + 2 * (size_t)row0 : nullptr, smem, a_alloc_rows);
@@ -559,11 +580,10 @@ __global__ __launch_bounds__(kThreads, 2) void expert_gemm_grouped_small_kernel(
                                                                                 const int* __restrict__ sched,
                                                                                 int n_col_tiles) {
     extern __shared__ __align__(16) float smem[];
-    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
-    const int first = sched[1 + xcd], share = sched[2 + xcd] - first;
-    if (slot >= share * n_col_tiles) return;
-    const RowTile rt = tiles[first + slot / n_col_tiles];
-    const int n0 = (slot % n_col_tiles) * BN;
+    RowTile rt;
+    int col_tile;
+    if (!grouped_slot(tiles, sched, n_col_tiles, &rt, &col_tile)) return;
+    const int n0 = col_tile * BN;
     const int owner = p.expert_slot ? p.expert_slot[rt.expert] : rt.expert;
     gemm_dispatch_small<BN, EPI>(p.A + (size_t)rt.row0 * p.K, p.R ? p.R + (size_t)rt.row0 * p.N : nullptr,
                                  p.C + (size_t)rt.row0 * p.N, rt.rows, p.B + (size_t)owner * weight_stride, n0, p.N, p.K,
