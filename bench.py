@@ -46,12 +46,15 @@ KERNEL_SOURCES = {
     "skinny": ("infmoe_amd/csrc/kernels/expert_skinny.hip",),
 }
 MEASURED_TRAFFIC = {
-    "c2": dict(ratio=5.77 / 5.60, kernel="gemm", source="profiles/c2_expert_gemm_grouped_kernel_stats.txt",
-               source_digest="unrecorded"),
-    "c5": dict(ratio=4.03 / 4.03, kernel="skinny", source="profiles/c5_expert_skinny_kernel_stats.txt",
-               source_digest="unrecorded"),
-    "c4": dict(ratio=7.90 / 4.97, kernel="gemm", source="profiles/c4_expert_gemm_grouped_kernel_stats.txt",
-               source_digest="unrecorded"),
+    # c2: 5.73 GB (mean of the two launches, fetched + written) against 5.60 GB of weights, rows and hidden rows
+    "c2": dict(ratio=5.726 / 5.604, kernel="gemm", source="profiles/c2_expert_gemm_grouped_kernel_stats.txt",
+               source_digest="b1d327d74c73"),
+    # c5: 4.70 GB against 4.70 GB of weights of the 28 active experts
+    "c5": dict(ratio=4.704 / 4.698, kernel="skinny", source="profiles/c5_expert_skinny_kernel_stats.txt",
+               source_digest="2e8ae4f7cbc5"),
+    # c4: 6.82 GB against 4.97 GB: the weights of an expert with several row tiles are fetched more than once
+    "c4": dict(ratio=6.820 / 4.966, kernel="gemm", source="profiles/c4_expert_gemm_grouped_kernel_stats.txt",
+               source_digest="b1d327d74c73"),
 }
 
 CONFIGS = {
@@ -415,6 +418,10 @@ def main():
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: only the headline workload (no decode shape, streamed configuration, "
                          "skewed workload, sweeps or vendor comparator)")
+    ap.add_argument("--legs", default="all",
+                    help="with the default workload: which of the further workloads to run, comma-separated, of "
+                         "c5,c2_uniform,vendor_bmm,sweep,c3,c4 (default all; e.g. c2_uniform,vendor_bmm to profile the two "
+                         "side by side)")
     ap.add_argument("--replicate-weights", action="store_true",
                     help="profiling aid: give every expert the values of expert 0 (short set-up, same work)")
     args = ap.parse_args()
@@ -502,7 +509,11 @@ def main():
     # Further workloads of the same run (the headline `value` above is untouched by them).
     secondary = {}
 
+    legs = None if args.legs == "all" else set(args.legs.split(","))
+
     def extra(key, fn):  # the headline line must not depend on the extras
+        if legs is not None and key not in legs:
+            return
         try:
             secondary[key] = fn()
         except Exception as exc:
@@ -550,6 +561,8 @@ def main():
         # this run, t_copy the streamed bytes at the bare rate of asynchronous copies of one slot
         def leg_c3():
             c3 = dict(CONFIGS["c3"], ffn=args.ffn)
+            if not slots:
+                raise RuntimeError("the streamed layer needs the host copies of the experts (not with --replicate-weights)")
             p3, x3, *_ = build_layer(torch, c3, keep_host=True, slots=slots)
             try:
                 steps3 = min(args.steps, 10)
