@@ -107,7 +107,8 @@ int32_t infmoe_set_score_bias(infmoe_plugin* p, const float* host);
 int32_t infmoe_configure(infmoe_plugin* p, const int32_t* dims, int32_t nb_dims);
 
 /* Replaces getWorkspaceSize (plugin/MoELayerPlugin.cc:253-273).  Bytes of caller-owned device
- * scratch infmoe_enqueue needs for an input of `dims`. */
+ * scratch infmoe_enqueue needs for an input of `dims`.  Never smaller for more tokens: a workspace sized for
+ * the largest batch serves every smaller one. */
 int32_t infmoe_workspace_size(const infmoe_plugin* p, const int32_t* dims, int32_t nb_dims, size_t* out_bytes);
 
 /* Replaces initialize (plugin/MoELayerPlugin.cc:197-201 -> plugin/sublayers/T5FFLayer.cc:143-147):
@@ -125,8 +126,10 @@ int32_t infmoe_initialize(infmoe_plugin* p);
  * Allocates nothing, neither device nor host memory, on either schedule (the lists the streamed schedule makes
  * per call live in the layer, sized by infmoe_initialize).
  *
- * Streams: the weight slots of a streamed layer (max_concurrency < expert_count) keep experts between calls, so a
- * call on another stream than the previous call's first waits, on the device, for that call's end.
+ * Streams: one infmoe_enqueue in flight per handle.  The weight slots of a streamed layer (max_concurrency <
+ * expert_count) keep experts between calls, so there a call on another stream than the previous call's first
+ * waits, on the device, for that call's end; with resident experts calls on different streams are the caller's
+ * to order (the layer's routing counts are one block of device memory).
  *
  * A token whose scores cannot be ordered (a NaN in its row; the reference asserts there,
  * plugin/cuda/moe.cu:70,184) does not stop the call, whatever the schedule: the call completes, that

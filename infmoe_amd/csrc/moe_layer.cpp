@@ -351,6 +351,11 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     int32_t* dOffset = dCount + E;
     int32_t* dStats = dOffset + E + 1;
 
+    // Streamed experts: the weight slots (and the routing block the host reads) outlive the call.  Work of an
+    // earlier call that uses them was joined into THAT call's stream; a call on another stream waits, on the
+    // device, for its end before it queues anything.
+    if (!resident() && mHaveCallDone && stream != mLastStream) INFMOE_HIP(hipStreamWaitEvent(stream, mCallDone, 0));
+
     const bool timed = mTiming && !mMarks.empty();
     hipEvent_t* marks = timed ? &mMarks[(size_t)(mTimedCalls % mTimingDepth) * (INFMOE_N_PHASES + 1)] : nullptr;
     auto mark = [&](int i) -> Status {
@@ -496,9 +501,6 @@ Status MoELayer::lastTiming(float* ms) {
 Status MoELayer::runStreamed(int T, const Carve& c, hipStream_t stream, GroupedRun& g) {
     const int E = mParams.expertCount, d = mParams.embeddingSize, mc = mParams.maxConcurrency;
     const size_t routingInts = (size_t)2 * E + 1 + 4;
-    // The slots outlive the call.  Work of an earlier call that reads or fills them was joined into THAT call's
-    // stream; a call on another stream waits for its end before it touches a slot.
-    if (mHaveCallDone && stream != mLastStream) INFMOE_HIP(hipStreamWaitEvent(stream, mCallDone, 0));
     INFMOE_HIP(hipMemcpyAsync(mRoutingHost, mRoutingGpu, sizeof(int32_t) * routingInts, hipMemcpyDeviceToHost, stream));
     INFMOE_HIP(hipStreamSynchronize(stream));
     const int32_t* count = mRoutingHost;

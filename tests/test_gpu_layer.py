@@ -647,3 +647,30 @@ def test_many_experts(torch_cuda, E, mc):
     y, ref, count, _ = run_and_check(torch_cuda, plugin, x, c, g, ws, shape, "cpm_2")
     assert count.sum() == 700 and (count > 0).sum() > E // 2
     plugin.terminate()
+
+
+def test_streamed_layer_called_from_alternating_streams(torch_cuda):
+    """The weight slots of a streamed layer outlive a call; a call on another stream than the last one's waits for
+    that call's end on the device.  Calls alternate between two streams without any host synchronisation in
+    between, each with its own buffers, and every output is the resident layer's, bit for bit."""
+    torch = torch_cuda
+    shape, E, d, h = (2, 96), 8, 64, 192
+    B, S = shape
+    resident, x, c, g, ws = make_layer(shape, E, d, h, E, "cpm_2", seed=97)
+    streamed, *_ = make_layer(shape, E, d, h, 3, "cpm_2", seed=97)
+    rng = np.random.default_rng(2)
+    inputs = [dev(torch, (x * s).reshape(B, S, d)) for s in (1.0, 0.5, 2.0, 1.5, 0.25, 3.0)]
+    want = [resident.forward(v).clone() for v in inputs]
+    torch.cuda.synchronize()
+    dims = [B, S, d]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.zeros_like(v) for v in inputs]
+    works = [torch.empty(streamed.workspace_size(dims), dtype=torch.uint8, device="cuda") for _ in streams]
+    for i, v in enumerate(inputs):
+        s = streams[i % 2]
+        streamed.enqueue(dims, v.data_ptr(), outs[i].data_ptr(), works[i % 2].data_ptr(), s.cuda_stream)
+    torch.cuda.synchronize()
+    for i in range(len(inputs)):
+        assert torch.equal(outs[i], want[i]), f"call {i} (stream {i % 2}) differs from the resident layer"
+    resident.terminate()
+    streamed.terminate()
