@@ -194,24 +194,36 @@ __global__ __launch_bounds__(kThreads, EPI == EPI_GATED_GELU ? 2 : 3) void exper
         B0 += (size_t)owner * weight_stride;
         if (GATED) B1 += (size_t)owner * weight_stride;
     }
+    if (rows <= 0) return;
+    // The last run of up to kSkinnyMaxRows rows - for nearly every expert of a decode call the only one - is
+    // straight-line code; the full runs of a taller expert go before it in a loop of the 8-row body.  (One loop
+    // over all runs around the switch cost the second product's kernel four spilled registers.)
+    const int last = ((rows - 1) / kSkinnyMaxRows) * kSkinnyMaxRows;  // first row of the last run
 #pragma unroll 1
-    for (; rows > 0; rows -= kSkinnyMaxRows, row0 += kSkinnyMaxRows) {  // (a body returns when its wave has no weight rows left)
-        const float* A = p.A + (size_t)row0 * p.K;
-        const float* R = p.R ? p.R + (size_t)row0 * p.N : nullptr;
-        float* C = p.C + (size_t)row0 * p.N;
-        const float* stats = EPI != EPI_RESIDUAL && p.row_stats != nullptr ? p.row_stats + 2 * (size_t)row0 : nullptr;
-        // One body per row count: a row more than needed would cost its loads of the activation chunk
-        // again for every block of weight rows (with 5 rows in the 8-row body, 60 % more of them).
-        switch (min(rows, kSkinnyMaxRows)) {
-            case 1: skinny_body<1, 8, 2, EPI>(A, R, C, 1, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 2: skinny_body<2, 8, 2, EPI>(A, R, C, 2, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 3: skinny_body<3, 2, 8, EPI>(A, R, C, 3, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 4: skinny_body<4, 2, 8, EPI>(A, R, C, 4, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 5: skinny_body<5, 1, 8, EPI>(A, R, C, 5, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 6: skinny_body<6, 1, 8, EPI>(A, R, C, 6, B0, B1, p.N, p.K, stats, row_blocks); break;
-            case 7: skinny_body<7, 1, 8, EPI>(A, R, C, 7, B0, B1, p.N, p.K, stats, row_blocks); break;
-            default: skinny_body<8, 1, 8, EPI>(A, R, C, 8, B0, B1, p.N, p.K, stats, row_blocks); break;
-        }
+    for (int r0 = 0; r0 < last; r0 += kSkinnyMaxRows) {  // (a body returns when its wave has no weight rows left)
+        const int at = row0 + r0;
+        skinny_body<8, 1, 8, EPI>(p.A + (size_t)at * p.K, p.R ? p.R + (size_t)at * p.N : nullptr, p.C + (size_t)at * p.N, 8,
+                                  B0, B1, p.N, p.K,
+                                  EPI != EPI_RESIDUAL && p.row_stats != nullptr ? p.row_stats + 2 * (size_t)at : nullptr,
+                                  row_blocks);
+    }
+    row0 += last;
+    rows -= last;
+    const float* A = p.A + (size_t)row0 * p.K;
+    const float* R = p.R ? p.R + (size_t)row0 * p.N : nullptr;
+    float* C = p.C + (size_t)row0 * p.N;
+    const float* stats = EPI != EPI_RESIDUAL && p.row_stats != nullptr ? p.row_stats + 2 * (size_t)row0 : nullptr;
+    // One body per row count: a row more than needed would cost its loads of the activation chunk
+    // again for every block of weight rows (with 5 rows in the 8-row body, 60 % more of them).
+    switch (rows) {
+        case 1: skinny_body<1, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 2: skinny_body<2, 8, 2, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 3: skinny_body<3, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 4: skinny_body<4, 2, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 5: skinny_body<5, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 6: skinny_body<6, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        case 7: skinny_body<7, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
+        default: skinny_body<8, 1, 8, EPI>(A, R, C, rows, B0, B1, p.N, p.K, stats, row_blocks); break;
     }
 }
 
