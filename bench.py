@@ -223,6 +223,18 @@ def cpu_baseline(cfg, x, cent, gamma, slots, bias, sample_tokens):
                       f"oracle/moe_cpu.c (FP32, OpenMP, AVX2), {dt:.2f} s"}
 
 
+def spin_up(torch, step, seconds=1.0):
+    """Untimed steps until `seconds` of wall time have passed: a part that comes out of idle takes a second or two of
+    load to settle its clocks (the reference's example stack ran 246, 239, 237 ms per step in three consecutive passes
+    of six steps), and a short run would otherwise report the settling.  Returns the number of steps."""
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        step()
+        torch.cuda.synchronize()
+        n += 1
+    return n
+
+
 def time_steps(torch, step, steps, warmup):
     """W untimed steps, then K timed ones with an event between every two of them (on torch's current stream,
     which is the stream `step` queues on).  Returns (per-step ms [K], ms from first to last event / K, host ms / K)."""
@@ -266,6 +278,7 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
             plugin.enqueue(dims, x.data_ptr(), y.data_ptr(), ws.data_ptr(), stream)
 
     plugin.set_timing(0)
+    settled = spin_up(torch, step)
     per_step, mean_ms, wall_ms = time_steps(torch, step, steps, warmup)
     plugin.set_timing(steps)
     marked_steps, marked_mean_ms, _ = time_steps(torch, step, steps, warmup)
@@ -333,7 +346,7 @@ def measure(torch, plugin, cfg, name, x, steps, warmup, gated=False, stack=None)
                        "frac_of_hbm_peak": round(v / (phases[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
                    for k, v in phase_bytes.items() if phases.get(k, 0) > 0}
     return dict(ms_per_step=float(np.median(per_step)), mean_ms=mean_ms, min_ms=float(np.min(per_step)),
-                marked_ms=float(np.median(marked_steps)), wall_ms=wall_ms, phases=phases, last=last, count=count,
+                marked_ms=float(np.median(marked_steps)), settled=settled, wall_ms=wall_ms, phases=phases, last=last, count=count,
                 stats=stats, active=active, resident=resident, roofline=roofline, phase_rates=phase_rates, tokens=T)
 
 
@@ -490,7 +503,9 @@ def main():
         "timing": {"value_from": "median of the per-step times of a pass with the library's phase marks off",
                    "ms_per_step_mean": round(m["mean_ms"], 4), "ms_per_step_min": round(m["min_ms"], 4),
                    "ms_per_step_with_phase_marks": round(m["marked_ms"], 4),
-                   "phases_from": "a second pass of the same length with the phase marks on"},
+                   "phases_from": "a second pass of the same length with the phase marks on",
+                   "untimed_steps_before_the_warmup": m["settled"],
+                   "why": "a second of load first, so that the part's clocks have settled when the W warm-up steps begin"},
         "roofline": roofline,
         "phases_ms": {k: round(v, 4) for k, v in phases.items()},
         "phases_ms_last_timed_step": {k: round(v, 4) for k, v in last.items()},
