@@ -62,13 +62,18 @@ def pick_experts(count, n, tile_rows):
     return list(dict.fromkeys(int(e) for e in picks))[:n]
 
 
-# the last case is the three-matrix form the reference's code computes, at c2's sizes
-@pytest.mark.parametrize("name,experts_to_check,ffn",
-                         [("c2", 6, "relu"), ("c5", 32, "relu"), ("c4", 6, "relu"), ("c2", 3, "gated_gelu")])
-def test_full_size_layer_whole_experts(lib, torch_cuda, name, experts_to_check, ffn):
+# the fourth case is the three-matrix form the reference's code computes, at c2's sizes; the last is the c2 layer on
+# the first 1024 tokens of its batch (21..46 rows per expert): the few-rows-per-expert form of the matrix-core kernel
+# in the grouped launch at the benchmark's widths
+@pytest.mark.parametrize("name,experts_to_check,ffn,tokens",
+                         [("c2", 6, "relu", 0), ("c5", 32, "relu", 0), ("c4", 6, "relu", 0), ("c2", 3, "gated_gelu", 0),
+                          ("c2", 8, "relu", 1024)])
+def test_full_size_layer_whole_experts(lib, torch_cuda, name, experts_to_check, ffn, tokens):
     torch = torch_cuda
     import bench
     cfg = dict(bench.CONFIGS[name], ffn=ffn)
+    if tokens:
+        cfg["shape"] = (tokens, 1)
     E, d, h = cfg["E"], cfg["d"], cfg["h"]
     B, S = cfg["shape"]
     T = B * S
@@ -94,7 +99,7 @@ def test_full_size_layer_whole_experts(lib, torch_cuda, name, experts_to_check, 
     # sample: which matrix instruction a row meets depends on its place in its row tile, and the tail
     # rows of a tile (16-row block, 4-row groups) only exist at the end of an expert's rows.
     yh = y.reshape(T, d).cpu().numpy()
-    tile_rows = 192 if ffn == "gated_gelu" else 256
+    tile_rows = 192 if ffn == "gated_gelu" else (96 if T <= 64 * E else 256)
     chosen = pick_experts(count, experts_to_check, tile_rows)
     checked = 0
     for e in chosen:
