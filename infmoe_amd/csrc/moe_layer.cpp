@@ -392,8 +392,8 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     g.maxTiles = std::min(c.maxTiles, max_row_tiles(T, E, mSublayer->rowTileHeightFor(T)));  // of this call's tile height
     if (skinnyMax > 0) {
         // Only experts with more than skinnyMax rows are cut into row tiles: at most T / (skinnyMax + 1)
-        // of them, each with one tile more than its rows fill.  A decode call then launches a small
-        // grid (or none) for the matrix-core kernel instead of one sized for E experts.
+        // of them, each with one tile more than its rows fill.  (T5_FF answers "every expert" for a decode call:
+        // no expert is tiled then and its grouped run launches no matrix-core grid at all.)
         const int tall = T / (skinnyMax + 1);
         g.maxTiles = std::min(g.maxTiles, tall + T / mSublayer->rowTileHeightFor(T));
     }
