@@ -355,6 +355,16 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
     // earlier call that uses them was joined into THAT call's stream; a call on another stream waits, on the
     // device, for its end before it queues anything.
     if (!resident() && mHaveCallDone && stream != mLastStream) INFMOE_HIP(hipStreamWaitEvent(stream, mCallDone, 0));
+    // ... and this call's end is marked on every way out of it, a failure halfway included: what it has queued
+    // by then uses the slots all the same.
+    struct CallEnd {
+        MoELayer* layer;
+        hipStream_t stream;
+        ~CallEnd() {
+            if (layer != nullptr && hipEventRecord(layer->mCallDone, stream) == hipSuccess)
+                layer->mHaveCallDone = true, layer->mLastStream = stream;
+        }
+    } callEnd{resident() ? nullptr : this, stream};
 
     const bool timed = mTiming && !mMarks.empty();
     hipEvent_t* marks = timed ? &mMarks[(size_t)(mTimedCalls % mTimingDepth) * (INFMOE_N_PHASES + 1)] : nullptr;
@@ -414,10 +424,6 @@ Status MoELayer::enqueue(const int32_t* dims, int32_t nbDims, const void* const*
         INFMOE_HIP(launch_gather(T, d, c.post, c.pos, y, stream, c.routedCoeff));
     INFMOE_TRY(mark(7));
     if (timed) ++mTimedCalls;
-    if (!grouped) {
-        INFMOE_HIP(hipEventRecord(mCallDone, stream));
-        mHaveCallDone = true, mLastStream = stream;
-    }
     if (!grouped && mNanRowsSeen > 0) {
         // reported here, not again by the next call (the routing was waited for, so the flag is this call's)
         __atomic_store_n(mNanFlagHost, 0, __ATOMIC_RELEASE);
